@@ -22,7 +22,7 @@ from typing import Dict, Hashable, List, Optional, Sequence as Seq, Tuple
 import numpy as np
 import torch
 
-from ..parts.base import KVRequirement, StateRequirement
+from ..parts.base import KVRequirement, StateRequirement, requirement_list
 from .pages import OutOfPages, PagePool
 from .state import StateSlots
 
@@ -36,23 +36,32 @@ def pages_for(tokens: int, page_size: int) -> int:
 def bytes_per_token(requirements: Seq[object], dtype: torch.dtype) -> int:
     """Cache bytes one token takes over all runs that keep keys and values."""
     elem = torch.empty((), dtype=dtype).element_size()
-    return sum(2 * r.n_kv_heads * r.head_dim * elem for r in requirements if isinstance(r, KVRequirement))
+    return sum(r.n_kv_heads * (r.head_dim + r.value_dim) * elem
+               for need in requirements for r in requirement_list(need) if isinstance(r, KVRequirement))
 
 
 def group_requirements(requirements: Seq[object]):
     """Runs by what they keep: ``({KVRequirement: [run ids]}`` in order of first appearance,
-    one entry per group of pages; ``{run id: StateRequirement})``."""
+    one entry per group of pages; ``{state key: StateRequirement})``.  A run may keep keys and
+    values and any number of states; a state's key is the run's id, or ``(run id, name)`` for a
+    state with a name."""
     by_need: Dict[KVRequirement, List[int]] = {}
-    states: Dict[int, StateRequirement] = {}
-    for cache_id, need in enumerate(requirements):
-        if need is None:
-            continue
-        if isinstance(need, KVRequirement):
-            by_need.setdefault(need, []).append(cache_id)
-        elif isinstance(need, StateRequirement):
-            states[cache_id] = need
-        else:
-            raise TypeError(f"run {cache_id} asks for an unknown kind of cache: {need!r}")
+    states: Dict[object, StateRequirement] = {}
+    for cache_id, needs in enumerate(requirements):
+        has_kv = False
+        for need in requirement_list(needs):
+            if isinstance(need, KVRequirement):
+                if has_kv:
+                    raise TypeError(f"run {cache_id} asks for two caches of keys and values")
+                has_kv = True
+                by_need.setdefault(need, []).append(cache_id)
+            elif isinstance(need, StateRequirement):
+                key = (cache_id, need.name) if need.name else cache_id
+                if key in states:
+                    raise TypeError(f"run {cache_id} asks for two states of one name: {need.name!r}")
+                states[key] = need
+            else:
+                raise TypeError(f"run {cache_id} asks for an unknown kind of cache: {need!r}")
     return by_need, states
 
 
@@ -112,11 +121,12 @@ class KVGroup:
         self.page_size = page_size
         self.pool = PagePool(num_pages)
         shape = (num_pages, page_size, requirement.n_kv_heads, requirement.head_dim)
+        v_shape = (num_pages, page_size, requirement.n_kv_heads, requirement.value_dim)
         # Same layout as the reference's pool (/root/reference/src/pylon/kv/pool.py:36-44):
         # page, slot in page, key/value head, element.  Zero-filled so that a slot no
         # token has written yet holds finite numbers.
         self.k: Dict[int, torch.Tensor] = {c: torch.zeros(shape, dtype=dtype, device=device) for c in cache_ids}
-        self.v: Dict[int, torch.Tensor] = {c: torch.zeros(shape, dtype=dtype, device=device) for c in cache_ids}
+        self.v: Dict[int, torch.Tensor] = {c: torch.zeros(v_shape, dtype=dtype, device=device) for c in cache_ids}
 
     def record_pages(self, slot: int, first_index: int, pages: List[int]) -> None:
         end = first_index + len(pages)
@@ -133,7 +143,7 @@ class KVGroup:
     def bytes_per_token(self) -> int:
         r = self.requirement
         elem = next(iter(self.k.values())).element_size() if self.k else 0
-        return len(self.cache_ids) * 2 * r.n_kv_heads * r.head_dim * elem
+        return len(self.cache_ids) * r.n_kv_heads * (r.head_dim + r.value_dim) * elem
 
 
 class Sequence:
@@ -161,6 +171,7 @@ class CacheView:
     block_table: Optional[torch.Tensor] = None  # int32 [rows, width]
     slot_map: Optional[torch.Tensor] = None  # int32 [tokens]: page * page_size + offset
     state: Optional[torch.Tensor] = None  # [max_slots, *shape] for stateful mixers
+    states: Optional[Dict[str, torch.Tensor]] = None  # the run's states that have a name
     group: int = -1
 
 
@@ -181,8 +192,11 @@ class CacheManager:
         self.group_of: Dict[int, int] = {}
         self.slots = StateSlots(max_requests)
         by_need, states = group_requirements(requirements)
-        for cache_id, need in states.items():
-            self.slots.add_state(cache_id, tuple(need.shape), need.dtype, device)
+        self._named_states: Dict[int, Dict[str, torch.Tensor]] = {}
+        for key, need in states.items():
+            tensor = self.slots.add_state(key, tuple(need.shape), need.dtype, device)
+            if need.name:
+                self._named_states.setdefault(key[0], {})[need.name] = tensor
         if isinstance(num_pages, int):
             per_group = [num_pages] * len(by_need)
         else:
@@ -362,13 +376,11 @@ class CacheManager:
 
     def view(self, cache_id: int) -> CacheView:
         """The storage side of a run's cache (tables and slot maps are added per step)."""
+        view = CacheView(state=self.slots.tensors.get(cache_id), states=self._named_states.get(cache_id))
         if cache_id in self.group_of:
             group = self.groups[self.group_of[cache_id]]
-            return CacheView(page_size=self.page_size, k=group.k[cache_id], v=group.v[cache_id],
-                             group=group.index)
-        if cache_id in self.slots.tensors:
-            return CacheView(state=self.slots.tensors[cache_id])
-        return CacheView()
+            view.page_size, view.k, view.v, view.group = self.page_size, group.k[cache_id], group.v[cache_id], group.index
+        return view
 
     # ---- invariants ---------------------------------------------------------------------
     def check(self) -> None:

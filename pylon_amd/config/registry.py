@@ -10,7 +10,7 @@ from __future__ import annotations
 import json
 from dataclasses import dataclass
 from pathlib import Path
-from typing import Callable, Dict, Mapping, Tuple
+from typing import Callable, Dict, Mapping, Optional, Tuple
 
 from .specs import ModelSpec
 
@@ -36,6 +36,9 @@ class Architecture:
     model_spec: Callable[[object], ModelSpec]
     weight_targets: Callable[[object], Dict[str, WeightTarget]]
     config_to_json: Callable[[object], dict]
+    # For a family in which some size is given only by a tensor's shape: the typed config
+    # completed from ``{tensor name: shape}`` of the model folder (headers only).
+    with_tensor_shapes: Optional[Callable[[object, Mapping], object]] = None
 
 
 _ARCHITECTURES: Dict[str, Architecture] = {}
@@ -57,6 +60,11 @@ def registered_architectures() -> Tuple[str, ...]:
 
 
 def architecture_name(config: Mapping) -> str:
+    """The name a config.json gives its model class: the one entry of ``architectures``, or the
+    string under ``architecture``."""
+    single = config.get("architecture")
+    if isinstance(single, str) and "architectures" not in config:
+        return single
     names = config.get("architectures")
     if not isinstance(names, (list, tuple)) or len(names) != 1 or not isinstance(names[0], str):
         raise ValueError(
@@ -92,7 +100,12 @@ def load_model_config(folder):
     """``(architecture, typed config)`` for the model folder ``folder``."""
     raw = read_config_json(folder)
     arch = resolve(raw)
-    return arch, arch.parse_config(raw)
+    config = arch.parse_config(raw)
+    if arch.with_tensor_shapes is not None:
+        from ..weights.loader import tensor_shapes
+
+        config = arch.with_tensor_shapes(config, tensor_shapes(folder))
+    return arch, config
 
 
 def read_stop_token_ids(folder) -> tuple:

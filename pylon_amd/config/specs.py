@@ -64,6 +64,77 @@ class AttentionSpec:
 
 
 @dataclass(frozen=True)
+class SinkAttentionSpec:
+    """Grouped-query softmax attention without rotation: positions enter as a learned bias by
+    distance, and the softmax has a sink (a key of score 0 without a value: one is added to the
+    denominator).  ``score = scale * q.k + rel[bucket(i - j), head]`` with ``bias_rows`` rows in
+    ``rel``: distances below ``bias_rows // 2`` have a row each, the other half of the rows
+    spreads logarithmically up to ``bias_far``, beyond which the last row is used.  Keys have
+    ``head_dim`` elements, values ``v_head_dim``."""
+
+    hidden_size: int
+    n_heads: int
+    n_kv_heads: int
+    head_dim: int
+    v_head_dim: int
+    scale: float
+    bias_rows: int
+    bias_far: float
+    sink: bool = True
+    window: Optional[int] = None
+    kind: str = "sink_attention"
+
+
+@dataclass(frozen=True)
+class RetentionSpec:
+    """Linear attention with one fixed decay per head and no softmax:
+    ``S_t = decay_h S_{t-1} + k_t v_t^T``, ``o_t = S_t^T q_t``; q and k are rotated by
+    ``position`` (k then multiplied by ``head_dim ** -0.5``), every head's ``o`` is divided by
+    its root mean square (``norm_eps`` inside the root), the heads are multiplied by
+    ``silu(W_g h)`` and projected."""
+
+    hidden_size: int
+    n_heads: int
+    head_dim: int
+    v_head_dim: int
+    decay: Tuple[float, ...]
+    position: PositionSpec
+    norm_eps: float
+    kind: str = "retention"
+
+
+@dataclass(frozen=True)
+class ShortConvSpec:
+    """``h + conv(h)``: a causal convolution of ``taps`` taps over time on each of ``dim``
+    channels, added to its input; a request's last ``taps - 1`` inputs are its state."""
+
+    dim: int
+    taps: int
+    kind: str = "short_conv"
+
+
+@dataclass(frozen=True)
+class CappedGatedFeedForwardSpec:
+    """``down(a(g) * (u + offset))`` with ``g = min(gate(x), limit)``, ``u = clamp(up(x), -limit,
+    limit)`` and ``a(g) = g * sigmoid(alpha * g)``; gate and up fused into one matrix."""
+
+    hidden_size: int
+    intermediate_size: int
+    limit: float
+    alpha: float = 1.702
+    offset: float = 1.0
+    kind: str = "capped_gated_mlp"
+
+
+@dataclass(frozen=True)
+class LogitScaleSpec:
+    """Logits times one constant."""
+
+    factor: float
+    kind: str = "scale"
+
+
+@dataclass(frozen=True)
 class GatedFeedForwardSpec:
     """``down(act(gate(x)) * up(x))`` with gate and up fused into one matrix."""
 
@@ -78,13 +149,19 @@ class LayerSpec:
     """One residual block: which mixer, which feed-forward, which norms, how arranged.
 
     ``arrangement="pre_norm"``: ``x += mixer(norm1(x)); x += ff(norm2(x))``.
+    ``arrangement="sandwich_norm"``: every sublayer is normed on both sides,
+    ``x += post1(mixer(conv(norm1(x)))); x += post2(ff(norm2(x)))``, where ``conv`` is the
+    optional ``input_conv`` in front of the mixer and ``feed_forward`` may be None.
     """
 
     mixer: object
     feed_forward: object
     mixer_norm: NormSpec
-    feed_forward_norm: NormSpec
+    feed_forward_norm: Optional[NormSpec]
     arrangement: str = "pre_norm"
+    mixer_post_norm: Optional[NormSpec] = None
+    feed_forward_post_norm: Optional[NormSpec] = None
+    input_conv: Optional[object] = None
 
     @property
     def kind(self) -> str:

@@ -5,6 +5,10 @@
 // maximum and sum in float, and accumulates the weighted values with one lane per
 // output element.  The walk starts at the first visible key of the token, so the order
 // of every sum depends only on the token's position and never on how the batch was cut.
+// Options: values of another size than keys; q rows that lie q_stride elements apart (a slice
+// of a fused projection); a learned bias by distance added to the scaled score,
+// rel[bucket[min(i - j, bucket_len - 1)] * n_heads + head]; and a sink, a key of score 0
+// without a value, which adds one to the softmax's denominator.
 #include "common.h"
 
 #define ATT_WAVES 4
@@ -49,7 +53,9 @@ __global__ void paged_attention_kernel(T* __restrict__ out, const T* __restrict_
                                        const int* __restrict__ block_table, int table_width,
                                        const int* __restrict__ tok_row, const int* __restrict__ positions,
                                        long long items, int n_heads, int n_kv_heads, int head_dim,
-                                       int page_size, int window, float scale) {
+                                       int page_size, int window, float scale, int v_dim, long long q_stride,
+                                       const float* __restrict__ rel, const int* __restrict__ bucket,
+                                       int bucket_len, int sink) {
   extern __shared__ float lds[];
   const int lane = threadIdx.x & (PYLON_WAVE - 1);
   const int wave = threadIdx.x / PYLON_WAVE;
@@ -60,7 +66,7 @@ __global__ void paged_attention_kernel(T* __restrict__ out, const T* __restrict_
   if (active) {
     t = static_cast<int>(item / n_heads);
     h = static_cast<int>(item - static_cast<long long>(t) * n_heads);
-    const T* qr = q + (static_cast<size_t>(t) * n_heads + h) * head_dim;
+    const T* qr = q + static_cast<size_t>(t) * q_stride + static_cast<size_t>(h) * head_dim;
     for (int i = lane; i < head_dim; i += PYLON_WAVE) qbuf[i] = to_float(qr[i]);
   }
   __syncthreads();
@@ -87,6 +93,10 @@ __global__ void paged_attention_kernel(T* __restrict__ out, const T* __restrict_
       float dot = 0.f;
       for (int d = 0; d < head_dim; d += 8) dot = Vec8<T>::dot(qbuf + d, kr + d, dot);
       s = dot * scale;
+      if (rel != nullptr) {
+        const int far = pos - j;
+        s += rel[static_cast<size_t>(bucket[far < bucket_len ? far : bucket_len - 1]) * n_heads + h];
+      }
     }
     const float m_new = fmaxf(m, wave_max(s));
     const float p = valid ? expf(s - m_new) : 0.f;
@@ -98,21 +108,22 @@ __global__ void paged_attention_kernel(T* __restrict__ out, const T* __restrict_
     for (int kk = 0; kk < count; ++kk) {
       const float pk = __shfl(p, kk, PYLON_WAVE);
       const int physk = __shfl(phys, kk, PYLON_WAVE);
-      const T* vr = v_cache + (static_cast<size_t>(physk) * n_kv_heads + kvh) * head_dim;
+      const T* vr = v_cache + (static_cast<size_t>(physk) * n_kv_heads + kvh) * v_dim;
 #pragma unroll
       for (int i = 0; i < DIMS_PER_LANE; ++i) {
         const int d = lane + PYLON_WAVE * i;
-        if (d < head_dim) acc[i] = fmaf(pk, to_float(vr[d]), acc[i]);
+        if (d < v_dim) acc[i] = fmaf(pk, to_float(vr[d]), acc[i]);
       }
     }
     m = m_new;
   }
-  T* orow = out + (static_cast<size_t>(t) * n_heads + h) * head_dim;
+  T* orow = out + (static_cast<size_t>(t) * n_heads + h) * v_dim;
+  if (sink) l += expf(-m);  // the sink's weight on the scale of the running maximum
   const float inv = 1.0f / l;
 #pragma unroll
   for (int i = 0; i < DIMS_PER_LANE; ++i) {
     const int d = lane + PYLON_WAVE * i;
-    if (d < head_dim) orow[d] = from_float<T>(acc[i] * inv);
+    if (d < v_dim) orow[d] = from_float<T>(acc[i] * inv);
   }
 }
 
@@ -120,8 +131,9 @@ template <typename T>
 static int launch_paged_attention(T* out, const T* q, const T* k_cache, const T* v_cache,
                                   const int* block_table, int table_width, const int* tok_row,
                                   const int* positions, int tokens, int n_heads, int n_kv_heads,
-                                  int head_dim, int page_size, int window, float scale,
-                                  hipStream_t stream) {
+                                  int head_dim, int page_size, int window, float scale, int v_dim,
+                                  long long q_stride, const float* rel, const int* bucket, int bucket_len,
+                                  int sink, hipStream_t stream) {
   const long long items = static_cast<long long>(tokens) * n_heads;
   const long long blocks = (items + ATT_WAVES - 1) / ATT_WAVES;
   dim3 grid((unsigned)blocks), block(ATT_WAVES * PYLON_WAVE);
@@ -129,12 +141,13 @@ static int launch_paged_attention(T* out, const T* q, const T* k_cache, const T*
 #define LAUNCH(DPL)                                                                                  \
   hipLaunchKernelGGL((paged_attention_kernel<T, DPL>), grid, block, lds, stream, out, q, k_cache,    \
                      v_cache, block_table, table_width, tok_row, positions, items, n_heads,          \
-                     n_kv_heads, head_dim, page_size, window, scale)
-  if (head_dim <= 64)
+                     n_kv_heads, head_dim, page_size, window, scale, v_dim, q_stride, rel, bucket,   \
+                     bucket_len, sink)
+  if (v_dim <= 64)
     LAUNCH(1);
-  else if (head_dim <= 128)
+  else if (v_dim <= 128)
     LAUNCH(2);
-  else if (head_dim <= 256)
+  else if (v_dim <= 256)
     LAUNCH(4);
   else
     LAUNCH(8);
@@ -142,7 +155,9 @@ static int launch_paged_attention(T* out, const T* q, const T* k_cache, const T*
   return 0;
 }
 
-// q, out: [tokens, n_heads, head_dim]. Caches: [pages*page_size, n_kv_heads, head_dim].
+// q: [tokens, n_heads, head_dim], rows q_stride elements apart; out: [tokens, n_heads, v_dim].
+// Caches: keys [pages*page_size, n_kv_heads, head_dim], values [pages*page_size, n_kv_heads, v_dim].
+// rel: null, or float [rows, n_heads] with bucket: int [bucket_len], every entry a row of rel.
 // block_table: [rows, table_width] page ids; tok_row[t] names the table row of token t;
 // positions[t] is the token's index in its request; keys first(t)..positions[t] are read,
 // first(t) = max(0, positions[t] - window + 1) when window > 0, else 0.
@@ -150,14 +165,19 @@ extern "C" int pylon_paged_attention(void* out, const void* q, const void* k_cac
                                      int dtype, const int* block_table, int table_width,
                                      const int* tok_row, const int* positions, int tokens, int n_heads,
                                      int n_kv_heads, int head_dim, int page_size, int window,
-                                     float scale, hipStream_t stream) {
+                                     float scale, int v_dim, long long q_stride, const float* rel,
+                                     const int* bucket, int bucket_len, int sink, hipStream_t stream) {
   PYLON_REQUIRE(pylon_valid_dtype(dtype), "paged_attention: unknown dtype");
   PYLON_REQUIRE(tokens >= 0 && n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
                 "paged_attention: %d query heads cannot be grouped over %d key/value heads", n_heads,
                 n_kv_heads);
-  PYLON_REQUIRE(head_dim >= 16 && head_dim % 16 == 0 && head_dim <= 512,
-                "paged_attention: head_dim %d must be a multiple of 16 between 16 and 512", head_dim);
+  PYLON_REQUIRE(head_dim >= 8 && head_dim % 8 == 0 && head_dim <= 512,
+                "paged_attention: head_dim %d must be a multiple of 8 between 8 and 512", head_dim);
   PYLON_REQUIRE(page_size > 0 && table_width > 0, "paged_attention: bad page size or table width");
+  PYLON_REQUIRE(v_dim >= 1 && v_dim <= 512, "paged_attention: values of 1 to 512 elements, got %d", v_dim);
+  PYLON_REQUIRE(q_stride >= static_cast<long long>(n_heads) * head_dim, "paged_attention: q rows overlap");
+  PYLON_REQUIRE(rel == nullptr || (bucket != nullptr && bucket_len >= 1),
+                "paged_attention: a bias by distance needs its table of buckets");
   PYLON_REQUIRE(window >= 0, "paged_attention: window must be 0 (none) or positive");
   if (tokens == 0) return 0;
   PYLON_REQUIRE(static_cast<long long>(tokens) * n_heads / ATT_WAVES < (1ll << 31),
@@ -165,11 +185,12 @@ extern "C" int pylon_paged_attention(void* out, const void* q, const void* k_cac
   if (dtype == PYLON_F32)
     launch_paged_attention<float>((float*)out, (const float*)q, (const float*)k_cache,
                                   (const float*)v_cache, block_table, table_width, tok_row, positions,
-                                  tokens, n_heads, n_kv_heads, head_dim, page_size, window, scale, stream);
+                                  tokens, n_heads, n_kv_heads, head_dim, page_size, window, scale, v_dim,
+                                  q_stride, rel, bucket, bucket_len, sink, stream);
   else
     launch_paged_attention<bf16_t>((bf16_t*)out, (const bf16_t*)q, (const bf16_t*)k_cache,
                                    (const bf16_t*)v_cache, block_table, table_width, tok_row, positions,
-                                   tokens, n_heads, n_kv_heads, head_dim, page_size, window, scale,
-                                   stream);
+                                   tokens, n_heads, n_kv_heads, head_dim, page_size, window, scale, v_dim,
+                                   q_stride, rel, bucket, bucket_len, sink, stream);
   PYLON_LAUNCHED("paged_attention");
 }

@@ -410,3 +410,61 @@ extern "C" int pylon_silu_gate(void* out, int out_dtype, const void* gate_up, in
 #undef GO
   PYLON_LAUNCHED("silu_gate");
 }
+
+// ---- gated activation with constants -----------------------------------------------------
+// out[t, i] = a(g) * (u + offset) with g = min(gu[t, i], limit), u = clamp(gu[t, inter + i], -limit,
+// limit) and a(g) = g / (1 + exp(-alpha * g)): a sigmoid-gated unit whose steepness, offset of
+// the linear branch and cap are the caller's (limit <= 0: no cap).
+template <typename TI, typename TO>
+__global__ void gated_act_kernel(TO* __restrict__ out, const TI* __restrict__ gu, int inter, size_t total,
+                                 float alpha, float offset, float limit) {
+  size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const size_t step = static_cast<size_t>(gridDim.x) * blockDim.x;
+  for (; i < total; i += step) {
+    const size_t t = i / inter;
+    const size_t c = i - t * inter;
+    float g = to_float(gu[t * 2 * inter + c]);
+    float u = to_float(gu[t * 2 * inter + inter + c]);
+    if (limit > 0.f) {
+      g = fminf(g, limit);
+      u = fminf(fmaxf(u, -limit), limit);
+    }
+    out[i] = from_float<TO>((g / (1.0f + expf(-alpha * g))) * (u + offset));
+  }
+}
+
+extern "C" int pylon_gated_act(void* out, int out_dtype, const void* gate_up, int in_dtype, int tokens, int inter,
+                               float alpha, float offset, float limit, hipStream_t stream) {
+  PYLON_REQUIRE(pylon_valid_dtype(in_dtype) && pylon_valid_dtype(out_dtype), "gated_act: unknown dtype");
+  PYLON_REQUIRE(tokens >= 0 && inter > 0, "gated_act: bad sizes tokens=%d inter=%d", tokens, inter);
+  const size_t total = static_cast<size_t>(tokens) * inter;
+  if (total == 0) return 0;
+  size_t blocks = (total + 255) / 256;
+  if (blocks > 65535u * 16u) blocks = 65535u * 16u;
+  dim3 grid((unsigned)blocks), block(256);
+#define GO(TI, TO)                                                                                             \
+  hipLaunchKernelGGL((gated_act_kernel<TI, TO>), grid, block, 0, stream, (TO*)out, (const TI*)gate_up, inter, \
+                     total, alpha, offset, limit)
+  if (in_dtype == PYLON_F32 && out_dtype == PYLON_F32) GO(float, float);
+  else if (in_dtype == PYLON_F32) GO(float, bf16_t);
+  else if (out_dtype == PYLON_F32) GO(bf16_t, float);
+  else GO(bf16_t, bf16_t);
+#undef GO
+  PYLON_LAUNCHED("gated_act");
+}
+
+// ---- scaling in place ------------------------------------------------------------------------
+__global__ void scale_kernel(float* __restrict__ x, size_t total, float factor) {
+  size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const size_t step = static_cast<size_t>(gridDim.x) * blockDim.x;
+  for (; i < total; i += step) x[i] *= factor;
+}
+
+extern "C" int pylon_scale(float* x, long long count, float factor, hipStream_t stream) {
+  PYLON_REQUIRE(count >= 0, "scale: negative count");
+  if (count == 0) return 0;
+  size_t blocks = (static_cast<size_t>(count) + 255) / 256;
+  if (blocks > 65535u * 16u) blocks = 65535u * 16u;
+  hipLaunchKernelGGL(scale_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, x, (size_t)count, factor);
+  PYLON_LAUNCHED("scale");
+}

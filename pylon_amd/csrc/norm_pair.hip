@@ -1,0 +1,109 @@
+// The residual sum of a layer whose sublayers are normed on both sides, fused with the norm
+// that follows it:
+//
+//   d = sum_p delta[p]                      (the sublayer's output, maybe as partial sums)
+//   x = resid + post_gain * d / rms(d)      (rms(v) = sqrt(mean(v^2) + eps); without post_gain: x = resid + d)
+//   out = gain * x / rms(x)                 (gain: one number, or one per element)
+//
+// All of it in float; `out` is rounded once on the store.  One workgroup per output row, the
+// row held in registers between the passes, so that a row costs one trip to memory.  The order
+// of every sum depends on the row's length and the workgroup's size only.
+#include "common.h"
+
+template <typename TD, typename TO, int PER>
+__global__ void add_normed_rmsnorm_kernel(TO* __restrict__ out, float* resid, const TD* __restrict__ delta,
+                                          int n_delta, long long delta_stride, const float* __restrict__ post_gain,
+                                          float post_eps, const float* __restrict__ gain, int gain_stride,
+                                          const int* __restrict__ row_idx, int dim, float eps, int write_resid) {
+  __shared__ float scratch[16];
+  const int r_out = blockIdx.x;
+  const int r_in = row_idx ? row_idx[r_out] : r_out;
+  float* xr = resid + static_cast<size_t>(r_in) * dim;
+  const TD* dr = delta ? delta + static_cast<size_t>(r_in) * dim : nullptr;
+  TO* yr = out + static_cast<size_t>(r_out) * dim;
+  float x[PER];
+  if (dr) {
+    float d[PER];
+    float ss = 0.f;
+#pragma unroll
+    for (int n = 0; n < PER; ++n) {
+      const int i = threadIdx.x + n * blockDim.x;
+      d[n] = 0.f;
+      if (i < dim) {
+        float v = to_float(dr[i]);
+        for (int p = 1; p < n_delta; ++p) v += to_float(dr[i + p * delta_stride]);
+        d[n] = v;
+        ss += v * v;
+      }
+    }
+    float mult = 1.0f;
+    if (post_gain) {
+      const float total = block_sum(ss, scratch);
+      mult = 1.0f / sqrtf(total / static_cast<float>(dim) + post_eps);
+    }
+    const float pg = post_gain ? post_gain[0] : 1.0f;
+#pragma unroll
+    for (int n = 0; n < PER; ++n) {
+      const int i = threadIdx.x + n * blockDim.x;
+      x[n] = 0.f;
+      if (i < dim) {
+        x[n] = xr[i] + (d[n] * mult) * pg;
+        if (write_resid) xr[i] = x[n];
+      }
+    }
+  } else {
+#pragma unroll
+    for (int n = 0; n < PER; ++n) {
+      const int i = threadIdx.x + n * blockDim.x;
+      x[n] = i < dim ? xr[i] : 0.f;
+    }
+  }
+  if (out == nullptr) return;
+  float ss = 0.f;
+#pragma unroll
+  for (int n = 0; n < PER; ++n) ss += x[n] * x[n];
+  const float total = block_sum(ss, scratch);
+  const float inv = 1.0f / sqrtf(total / static_cast<float>(dim) + eps);
+#pragma unroll
+  for (int n = 0; n < PER; ++n) {
+    const int i = threadIdx.x + n * blockDim.x;
+    if (i < dim) yr[i] = from_float<TO>((x[n] * inv) * gain[static_cast<size_t>(i) * gain_stride]);
+  }
+}
+
+// resid: float [tokens, dim], updated in place unless row_idx picks rows.  delta: null (nothing
+// is added), [tokens, dim], or n_delta such tensors delta_stride elements apart.  post_gain: null
+// (delta is added as it is) or one float.  gain: one float (gain_stride 0) or dim floats
+// (gain_stride 1).  out: [rows, dim] of out_dtype, or null (only the sum is formed).
+extern "C" int pylon_add_normed_rmsnorm(void* out, int out_dtype, float* resid, const void* delta, int delta_dtype,
+                                        int n_delta, long long delta_stride, const float* post_gain, float post_eps,
+                                        const float* gain, int gain_stride, const int* row_idx, int rows, int dim,
+                                        float eps, hipStream_t stream) {
+  PYLON_REQUIRE(pylon_valid_dtype(out_dtype) && pylon_valid_dtype(delta_dtype), "add_normed_rmsnorm: unknown dtype");
+  PYLON_REQUIRE(rows >= 0 && dim > 0 && dim <= 16384, "add_normed_rmsnorm: rows of 1 to 16384 elements, got %d", dim);
+  PYLON_REQUIRE(n_delta >= 1 && (gain_stride == 0 || gain_stride == 1), "add_normed_rmsnorm: bad delta count or gain stride");
+  PYLON_REQUIRE(out == nullptr || gain != nullptr, "add_normed_rmsnorm: a norm needs its gain");
+  PYLON_REQUIRE(out != nullptr || (delta != nullptr && row_idx == nullptr), "add_normed_rmsnorm: nothing to do");
+  if (rows == 0) return 0;
+  const int write_resid = row_idx == nullptr ? 1 : 0;
+  const int threads = dim <= 256 ? 64 : (dim <= 2048 ? 256 : (dim <= 8192 ? 512 : 1024));
+  const int per = (dim + threads - 1) / threads;
+  dim3 grid(rows), block(threads);
+#define GO(TD, TO, PER)                                                                                         \
+  hipLaunchKernelGGL((add_normed_rmsnorm_kernel<TD, TO, PER>), grid, block, 0, stream, (TO*)out, resid,         \
+                     (const TD*)delta, n_delta, delta_stride, post_gain, post_eps, gain, gain_stride, row_idx,  \
+                     dim, eps, write_resid)
+#define PICK(TD, TO)            \
+  do {                          \
+    if (per <= 4) GO(TD, TO, 4);      \
+    else if (per <= 8) GO(TD, TO, 8); \
+    else GO(TD, TO, 16);        \
+  } while (0)
+  if (delta_dtype == PYLON_F32 && out_dtype == PYLON_F32) PICK(float, float);
+  else if (delta_dtype == PYLON_F32) PICK(float, bf16_t);
+  else if (out_dtype == PYLON_F32) PICK(bf16_t, float);
+  else PICK(bf16_t, bf16_t);
+#undef PICK
+#undef GO
+  PYLON_LAUNCHED("add_normed_rmsnorm");
+}

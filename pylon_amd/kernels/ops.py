@@ -188,14 +188,26 @@ def qkv_prepare(qkv: torch.Tensor, q_out: torch.Tensor, k_cache: Optional[torch.
 def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                     block_table: torch.Tensor, tok_row: torch.Tensor, positions: torch.Tensor, *,
                     page_size: int, window: Optional[int], scale: float,
-                    out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Causal attention of each token over its request's cached keys ``<=`` its position."""
+                    out: Optional[torch.Tensor] = None, rel: Optional[torch.Tensor] = None,
+                    bucket: Optional[torch.Tensor] = None, sink: bool = False) -> torch.Tensor:
+    """Causal attention of each token over its request's cached keys ``<=`` its position.
+    ``q`` is ``[tokens, heads, head_dim]`` and may be a slice of wider rows (a fused
+    projection); values may have another size than keys.  ``rel`` (float32 ``[rows, heads]``)
+    with ``bucket`` (int32 ``[n]``) adds ``rel[bucket[min(i - j, n - 1)], head]`` to the scaled
+    score of query ``i`` and key ``j``; ``sink`` adds one to the softmax's denominator."""
     if q.dim() != 3:
         raise KernelError("paged_attention takes q as [tokens, heads, head_dim]")
     tokens, n_heads, head_dim = q.shape
-    if k_cache.dim() != 4 or k_cache.shape != v_cache.shape:
+    if k_cache.dim() != 4 or v_cache.dim() != 4 or k_cache.shape[:3] != v_cache.shape[:3]:
         raise KernelError("paged_attention: caches must be [pages, page_size, kv_heads, head_dim]")
     pages, psize, n_kv_heads, hd = k_cache.shape
+    v_dim = v_cache.shape[3]
+    if q.stride(2) != 1 or q.stride(1) != head_dim or (tokens > 1 and q.stride(0) < n_heads * head_dim):
+        raise KernelError("paged_attention: the heads of a q row must lie side by side")
+    if (rel is None) != (bucket is None):
+        raise KernelError("paged_attention: rel and bucket go together")
+    if rel is not None and (rel.dim() != 2 or rel.shape[1] != n_heads or bucket.numel() < 1):
+        raise KernelError("paged_attention: rel must be [rows, heads] and bucket hold at least one entry")
     if psize != page_size or hd != head_dim:
         raise KernelError("paged_attention: cache geometry does not match page_size/head_dim")
     if k_cache.dtype != q.dtype or v_cache.dtype != q.dtype:
@@ -207,15 +219,151 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     if tok_row.numel() != tokens or positions.numel() != tokens:
         raise KernelError("paged_attention: one row id and one position per token are required")
     if out is None:
-        out = torch.empty_like(q)
-    elif out.shape != q.shape or out.dtype != q.dtype:
+        out = torch.empty((tokens, n_heads, v_dim), dtype=q.dtype, device=q.device)
+    elif out.shape != (tokens, n_heads, v_dim) or out.dtype != q.dtype:
         raise KernelError("paged_attention: out has the wrong shape or dtype")
-    _lib.call("pylon_paged_attention", _dev(out, "out"), _dev(q, "q"), _dev(k_cache, "k_cache"),
+    if not q.is_cuda:
+        raise KernelError("q must live on the GPU; there is no CPU path")
+    _lib.call("pylon_paged_attention", _dev(out, "out"), q.data_ptr(), _dev(k_cache, "k_cache"),
               _dev(v_cache, "v_cache"), dtype_code(q.dtype), _dev(block_table, "block_table", torch.int32),
               block_table.shape[1], _dev(tok_row, "tok_row", torch.int32),
               _dev(positions, "positions", torch.int32), tokens, n_heads, n_kv_heads, head_dim,
-              page_size, int(window or 0), float(scale), _stream())
+              page_size, int(window or 0), float(scale), v_dim, q.stride(0) if tokens > 1 else n_heads * head_dim,
+              _dev(rel, "rel", torch.float32), _dev(bucket, "bucket", torch.int32),
+              0 if bucket is None else bucket.numel(), 1 if sink else 0, _stream())
     return out
+
+
+def add_normed_rmsnorm(resid: torch.Tensor, delta: Optional[torch.Tensor], gain: Optional[torch.Tensor], eps: float,
+                       out_dtype: Optional[torch.dtype], *, post_gain: Optional[torch.Tensor] = None,
+                       post_eps: float = 0.0, row_idx: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """``resid += post_gain * d / rms(d)`` (``d`` = ``delta``, or the sum of a stack of float32
+    partial sums; without ``post_gain``: ``resid += d``), in float32 and in place, then
+    ``gain * resid / rms(resid)`` in ``out_dtype``, with ``rms(v) = sqrt(mean(v^2) + eps)``.
+    ``post_gain`` is one float32 number on the device; ``gain`` one number or one per element.
+    With ``row_idx`` only those rows are normed and ``resid`` is left as it is; with
+    ``gain`` None only the sum is formed."""
+    if resid.dim() != 2:
+        raise KernelError("add_normed_rmsnorm takes a 2-D residual")
+    dim = resid.shape[1]
+    n_delta, delta_stride = 1, 0
+    if delta is not None:
+        if delta.dim() == 3:
+            n_delta, delta_stride = delta.shape[0], delta.shape[1] * delta.shape[2]
+            if delta.shape[1:] != resid.shape:
+                raise KernelError("add_normed_rmsnorm: partial sums and resid differ in shape")
+        elif delta.shape != resid.shape:
+            raise KernelError("add_normed_rmsnorm: delta and resid differ in shape")
+    if post_gain is not None and post_gain.numel() != 1:
+        raise KernelError("add_normed_rmsnorm: post_gain is one number")
+    gain_stride = 0
+    if gain is not None:
+        if gain.numel() == dim and gain.dim() == 1 and dim > 1:
+            gain_stride = 1
+        elif gain.numel() != 1:
+            raise KernelError(f"add_normed_rmsnorm: gain must be one number or ({dim},)")
+    rows = resid.shape[0] if row_idx is None else row_idx.numel()
+    out = None
+    if gain is not None:
+        out = torch.empty((rows, dim), dtype=out_dtype, device=resid.device)
+    _lib.call("pylon_add_normed_rmsnorm", _dev(out, "out"), dtype_code(out.dtype) if out is not None else F32,
+              _dev(resid, "resid", torch.float32), _dev(delta, "delta"),
+              dtype_code(delta.dtype) if delta is not None else F32, n_delta, delta_stride,
+              _dev(post_gain, "post_gain", torch.float32), float(post_eps), _dev(gain, "gain", torch.float32),
+              gain_stride, _dev(row_idx, "row_idx", torch.int32), rows, dim, float(eps), _stream())
+    return out
+
+
+def short_conv(h: torch.Tensor, weight: torch.Tensor, state: Optional[torch.Tensor], row_start: torch.Tensor,
+               row_slots: torch.Tensor, *, rows: int, max_count: int, out_dtype: torch.dtype) -> torch.Tensor:
+    """``h[t] + sum_j weight[:, j] * h[t - taps + 1 + j]`` per channel and request, zeros before a
+    request's start.  ``state`` (float32 ``[slots, taps - 1, width]``) holds every request's last
+    ``taps - 1`` inputs and is brought up to date; ``max_count`` bounds the tokens of a row."""
+    if h.dim() != 2 or weight.dim() != 2 or weight.shape[0] != h.shape[1]:
+        raise KernelError("short_conv takes h [tokens, width] and weight [width, taps]")
+    tokens, width = h.shape
+    taps = weight.shape[1]
+    if taps > 1 and (state is None or state.dim() != 3 or state.shape[1:] != (taps - 1, width)):
+        raise KernelError(f"short_conv: state must be [slots, {taps - 1}, {width}]")
+    if row_start.numel() != rows + 1 or row_slots.numel() != rows:
+        raise KernelError("short_conv: one start per row and one more, and one slot per row")
+    out = torch.empty((tokens, width), dtype=out_dtype, device=h.device)
+    _lib.call("pylon_short_conv", _dev(out, "out"), dtype_code(out_dtype), _dev(h, "h"), dtype_code(h.dtype),
+              _dev(weight, "weight"), dtype_code(weight.dtype), _dev(state, "state", torch.float32),
+              _dev(row_start, "row_start", torch.int32), _dev(row_slots, "row_slots", torch.int32), rows,
+              int(max_count), width, taps, _stream())
+    return out
+
+
+def retention_recurrent(proj: torch.Tensor, state: torch.Tensor, decay: torch.Tensor,
+                        inv_freq: Optional[torch.Tensor], positions: torch.Tensor, row_start: torch.Tensor,
+                        row_slots: torch.Tensor, *, rows: int, heads: int, dim: int, vdim: int, rot_dims: int,
+                        eps: float, k_scale: float) -> torch.Tensor:
+    """Retention, token by token: ``proj`` ``[tokens, 2 heads dim + 2 heads vdim]`` holds q, k, v
+    and the gate side by side; ``state`` (float32 ``[slots, heads, dim, vdim]``) is read and left
+    up to date.  Returns the gated, per-head normalised output ``[tokens, heads * vdim]``."""
+    if proj.dim() != 2 or proj.shape[1] != 2 * heads * dim + 2 * heads * vdim or proj.stride(1) != 1:
+        raise KernelError("retention: the projection's rows must hold q, k, v and the gate")
+    tokens = proj.shape[0]
+    if state.dim() != 4 or state.shape[1:] != (heads, dim, vdim):
+        raise KernelError(f"retention: state must be [slots, {heads}, {dim}, {vdim}]")
+    if decay.numel() != heads or positions.numel() != tokens:
+        raise KernelError("retention: one decay per head and one position per token")
+    if row_start.numel() != rows + 1 or row_slots.numel() != rows:
+        raise KernelError("retention: one start per row and one more, and one slot per row")
+    if rot_dims and (inv_freq is None or inv_freq.numel() != rot_dims // 2):
+        raise KernelError("retention: inv_freq must hold rot_dims/2 frequencies")
+    if not proj.is_cuda:
+        raise KernelError("proj must live on the GPU; there is no CPU path")
+    out = torch.empty((tokens, heads * vdim), dtype=proj.dtype, device=proj.device)
+    _lib.call("pylon_retention_recurrent", _dev(out, "out"), proj.data_ptr(), dtype_code(proj.dtype), proj.stride(0),
+              0, heads * dim, 2 * heads * dim, 2 * heads * dim + heads * vdim, _dev(state, "state", torch.float32),
+              _dev(decay, "decay", torch.float32), _dev(inv_freq, "inv_freq", torch.float32), int(rot_dims),
+              _dev(positions, "positions", torch.int32), _dev(row_start, "row_start", torch.int32),
+              _dev(row_slots, "row_slots", torch.int32), rows, heads, dim, vdim, float(eps), float(k_scale),
+              _stream())
+    return out
+
+
+def kv_store(proj: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, slot_map: torch.Tensor, *,
+             k_off: int, v_off: int) -> None:
+    """Copy every token's keys (``proj[t, k_off:]``) and values (``proj[t, v_off:]``) into its
+    cache slot; the caches are ``[pages, page_size, kv_heads, size]`` with sizes of their own."""
+    if proj.dim() != 2 or proj.stride(1) != 1 or k_cache.dim() != 4 or v_cache.dim() != 4:
+        raise KernelError("kv_store takes a 2-D projection and 4-D caches")
+    if k_cache.dtype != proj.dtype or v_cache.dtype != proj.dtype:
+        raise KernelError("kv_store: the projection and the caches differ in dtype")
+    tokens = proj.shape[0]
+    if slot_map.numel() != tokens:
+        raise KernelError("kv_store: one cache slot per token is required")
+    k_row, v_row = k_cache.shape[2] * k_cache.shape[3], v_cache.shape[2] * v_cache.shape[3]
+    if max(k_off + k_row, v_off + v_row) > proj.shape[1]:
+        raise KernelError("kv_store: keys or values lie outside the projection's rows")
+    if not proj.is_cuda:
+        raise KernelError("proj must live on the GPU; there is no CPU path")
+    _lib.call("pylon_kv_store", _dev(k_cache, "k_cache"), _dev(v_cache, "v_cache"), proj.data_ptr(),
+              dtype_code(proj.dtype), proj.stride(0), int(k_off), int(v_off), _dev(slot_map, "slot_map", torch.int32),
+              tokens, k_row, v_row, _stream())
+
+
+def gated_act(gate_up: torch.Tensor, *, alpha: float, offset: float, limit: float,
+              out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """``a(g) * (u + offset)`` for a ``[tokens, 2I]`` input holding ``g`` then ``u``, with
+    ``a(g) = g * sigmoid(alpha * g)``, ``g`` capped from above at ``limit`` and ``u`` to
+    ``[-limit, limit]`` (``limit <= 0``: no cap).  float32 sums in, bfloat16 out: one rounding."""
+    if gate_up.dim() != 2 or gate_up.shape[1] % 2:
+        raise KernelError("gated_act takes a [tokens, 2*I] input")
+    tokens, two_i = gate_up.shape
+    out = torch.empty((tokens, two_i // 2), dtype=out_dtype or gate_up.dtype, device=gate_up.device)
+    _lib.call("pylon_gated_act", _dev(out, "out"), dtype_code(out.dtype), _dev(gate_up, "gate_up"),
+              dtype_code(gate_up.dtype), tokens, two_i // 2, float(alpha), float(offset), float(limit), _stream())
+    return out
+
+
+def scale_(x: torch.Tensor, factor: float) -> torch.Tensor:
+    """``x *= factor`` in place (float32)."""
+    _lib.call("pylon_scale", _dev(x, "x", torch.float32), x.numel(), float(factor), _stream())
+    return x
 
 
 DECODE_HEAD_DIMS = (64, 128, 256)

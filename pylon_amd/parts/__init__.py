@@ -1,12 +1,14 @@
 """The parts layers are assembled from; importing this package registers the built-in ones."""
-from . import attention, block, feed_forward, norm, position  # noqa: F401
-from .base import KVRequirement, Part, StateRequirement, summed
+from . import attention, block, feed_forward, logits, norm, position, retention, short_conv  # noqa: F401
+from .base import KVRequirement, Normed, Part, StateRequirement, requirement_list, summed
 from .registry import build_part, register_part, registered, unregister_part
 
 __all__ = [
     "KVRequirement",
     "StateRequirement",
     "Part",
+    "Normed",
+    "requirement_list",
     "summed",
     "build_part",
     "register_part",

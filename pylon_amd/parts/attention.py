@@ -11,7 +11,9 @@ from __future__ import annotations
 
 import torch
 
-from ..config.specs import AttentionSpec
+import math
+
+from ..config.specs import AttentionSpec, SinkAttentionSpec
 from ..kernels import ops
 from .base import KVRequirement, Part
 from .registry import build_part, register_part
@@ -126,4 +128,69 @@ class Attention(Part):
                                        out_dtype=self.dtype)
 
 
+def distance_buckets(rows: int, far: float) -> list:
+    """Row of a bias table of ``rows`` rows for every distance from 0 up to the first one that
+    is at least ``far``: distances below ``rows // 2`` have a row each; from there on
+    ``half + floor(log(n / half) / log(far / half) * (rows - half))``, capped at the last row,
+    which every distance of at least ``far`` reaches.  Computed once, in double precision."""
+    half = rows // 2
+    if rows < 2 or not far > half:
+        raise ValueError(f"a bias table of {rows} rows cannot spread its second half up to distance {far}")
+    out = []
+    for n in range(int(math.ceil(far)) + 1):
+        if n < half:
+            out.append(n)
+        else:
+            out.append(min(rows - 1, half + int(math.floor(math.log(n / half) / math.log(far / half) * (rows - half)))))
+    return out
+
+
+class SinkAttention(Part):
+    """Grouped-query attention over the paged cache with a learned bias by distance in place
+    of a rotation, a sink in the softmax's denominator, and values of another size than keys.
+    ``[q; k; v] = W h`` in one product; k and v go to the tokens' cache slots as they are;
+    scores, bias and softmax are float32."""
+
+    def __init__(self, spec: SinkAttentionSpec, *, dtype: torch.dtype, device) -> None:
+        super().__init__()
+        if spec.n_heads % spec.n_kv_heads:
+            raise ValueError("The number of Q heads must be divisible by the number of KV heads.")
+        if spec.head_dim % 8 or not 8 <= spec.head_dim <= 512 or not 1 <= spec.v_head_dim <= 512:
+            raise ValueError(f"heads of {spec.head_dim} key and {spec.v_head_dim} value elements are not supported: "
+                             "keys take multiples of 8 up to 512, values 1 to 512")
+        if spec.window is not None and spec.window < 1:
+            raise ValueError("window must be positive (or None for full attention)")
+        self.spec = spec
+        self.dtype = dtype
+        self.q_size = spec.n_heads * spec.head_dim
+        self.k_size = spec.n_kv_heads * spec.head_dim
+        self.v_size = spec.n_kv_heads * spec.v_head_dim
+        self.add_param("qkv", (self.q_size + self.k_size + self.v_size, spec.hidden_size), dtype, device)
+        self.add_param("out", (spec.hidden_size, spec.n_heads * spec.v_head_dim), dtype, device)
+        self.add_param("rel", (spec.bias_rows, spec.n_heads), torch.float32, device, role="vector")
+        self.bucket = torch.tensor(distance_buckets(spec.bias_rows, spec.bias_far), dtype=torch.int32).to(device)
+
+    def cache_requirement(self) -> KVRequirement:
+        spec = self.spec
+        return KVRequirement(spec.n_kv_heads, spec.head_dim, spec.window, v_head_dim=spec.v_head_dim)
+
+    def decode_signature(self, rows: int, bound: int) -> tuple:
+        return ("sink_attention",)  # one wave per (token, head), whatever the lengths
+
+    def forward(self, h: torch.Tensor, ctx, cache, stores: bool) -> torch.Tensor:
+        spec = self.spec
+        tokens = h.shape[0]
+        weight = self.params["qkv"] if stores else self.params["qkv"][: self.q_size]
+        qkv = ops.linear(h, weight, out_dtype=self.dtype)
+        if stores:
+            ops.kv_store(qkv, cache.k, cache.v, cache.slot_map, k_off=self.q_size, v_off=self.q_size + self.k_size)
+        q = qkv[:, : self.q_size].view(tokens, spec.n_heads, spec.head_dim)
+        context = ops.paged_attention(
+            q, cache.k, cache.v, cache.block_table, ctx.tok_row, ctx.positions, page_size=cache.page_size,
+            window=spec.window, scale=spec.scale, rel=self.params["rel"], bucket=self.bucket, sink=spec.sink)
+        return ops.linear_for_residual(context.view(tokens, spec.n_heads * spec.v_head_dim), self.params["out"],
+                                       out_dtype=self.dtype)
+
+
 register_part("mixer", "attention", Attention, replace=True)
+register_part("mixer", "sink_attention", SinkAttention, replace=True)

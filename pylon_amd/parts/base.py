@@ -10,13 +10,14 @@ norm          ``forward(x) -> y`` and ``add_forward(resid, delta, row_idx=None) 
               ``resid`` is the float32 residual stream, ``delta`` the previous part's
               output (or None), either ``[tokens, dim]`` or a stack ``[parts, tokens, dim]``
               of float32 partial sums still to be added up (:func:`summed` makes one float32
-              tensor of either); the sum is formed in float32, stored back into
+              tensor of either), or a :class:`Normed` (such an output that is normed before it
+              is added); the sum is formed in float32, stored back into
               ``resid`` (unless ``row_idx`` picks rows), and its norm is returned in
               the activation dtype.
 position      ``rotary() -> (inv_freq, rotary_dim) | None`` for encodings applied by
               rotating q and k: float32 frequencies of the pairs ``(i, i + rotary_dim/2)``
               of the first ``rotary_dim`` elements of a head; None encodes nothing.
-mixer         ``cache_requirement() -> KVRequirement | StateRequirement | None`` and
+mixer         ``cache_requirement() -> KVRequirement | StateRequirement | a tuple of them | None`` and
               ``forward(h, ctx, cache, stores) -> [tokens, hidden]`` (or partial sums
               ``[parts, tokens, hidden]`` in float32, see norm): ``cache`` is the
               view of the run's cache (its own, or the one it borrows); ``stores``
@@ -47,14 +48,44 @@ class KVRequirement:
     n_kv_heads: int
     head_dim: int
     window: Optional[int] = None  # keep only the last `window` tokens' entries
+    v_head_dim: Optional[int] = None  # size of a value head where it differs from a key head's
+
+    @property
+    def value_dim(self) -> int:
+        return self.head_dim if self.v_head_dim is None else self.v_head_dim
 
 
 @dataclass(frozen=True)
 class StateRequirement:
-    """Per-request state of fixed size, overwritten in place by every step."""
+    """Per-request state of fixed size, overwritten in place by every step.  A run that keeps
+    several states (or one beside its keys and values) gives each a ``name``; the run's cache
+    view then holds it as ``states[name]``."""
 
     shape: Tuple[int, ...]
     dtype: torch.dtype = torch.float32
+    name: str = ""
+
+
+def requirement_list(need) -> Tuple[object, ...]:
+    """What a run keeps, as a tuple: ``cache_requirement()`` may return nothing, one
+    requirement, or several (at most one of them keys and values)."""
+    if need is None:
+        return ()
+    if isinstance(need, (KVRequirement, StateRequirement)):
+        return (need,)
+    return tuple(need)
+
+
+@dataclass
+class Normed:
+    """A part's output that is still to be divided by its root mean square (``eps`` inside the
+    root), multiplied by ``gain`` (one float32 number on the device) and added to the residual
+    stream: what a layer that norms its sublayers on both sides hands to the next norm.
+    ``value`` is ``[tokens, dim]`` or a stack ``[parts, tokens, dim]`` of float32 partial sums."""
+
+    value: torch.Tensor
+    gain: torch.Tensor
+    eps: float
 
 
 def summed(delta: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
@@ -66,6 +97,10 @@ def summed(delta: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
     through this function (the built-in norm kernel takes both forms directly)."""
     if delta is None:
         return None
+    if isinstance(delta, Normed):
+        value = summed(delta.value)
+        rms = torch.sqrt(value.square().mean(dim=-1, keepdim=True) + delta.eps)
+        return value / rms * delta.gain.float()
     return delta.sum(dim=0) if delta.dim() == 3 else delta.float()
 
 

@@ -4,7 +4,7 @@ from __future__ import annotations
 
 import torch
 
-from ..config.specs import GatedFeedForwardSpec
+from ..config.specs import CappedGatedFeedForwardSpec, GatedFeedForwardSpec
 from ..kernels import ops, plan
 from .base import Part
 from .registry import register_part
@@ -27,4 +27,28 @@ class GatedFeedForward(Part):
         return ops.linear_for_residual(hidden, self.params["down"], out_dtype=self.dtype)
 
 
+class CappedGatedFeedForward(Part):
+    """``down(a(g) * (u + offset))``, ``g = min(gate(h), limit)``, ``u = clamp(up(h), -limit,
+    limit)``, ``a(g) = g * sigmoid(alpha * g)``.  As in the plain gated feed-forward, up to 128
+    rows the activation works on the float32 sums of the product and its result is rounded
+    once; beyond, the library's product is rounded first."""
+
+    def __init__(self, spec: CappedGatedFeedForwardSpec, *, dtype: torch.dtype, device) -> None:
+        super().__init__()
+        self.spec = spec
+        self.dtype = dtype
+        element_size = torch.empty((), dtype=dtype).element_size()
+        self.add_param("gate_up", (2 * spec.intermediate_size, spec.hidden_size), dtype, device,
+                       row_padding=plan.gated_row_padding(spec.hidden_size, element_size))
+        self.add_param("down", (spec.hidden_size, spec.intermediate_size), dtype, device)
+
+    def forward(self, h: torch.Tensor, ctx) -> torch.Tensor:
+        spec = self.spec
+        sums = torch.float32 if h.shape[0] <= ops.SPLIT_ROWS else self.dtype
+        gate_up = ops.linear(h, self.params["gate_up"], out_dtype=sums)
+        hidden = ops.gated_act(gate_up, alpha=spec.alpha, offset=spec.offset, limit=spec.limit, out_dtype=self.dtype)
+        return ops.linear_for_residual(hidden, self.params["down"], out_dtype=self.dtype)
+
+
 register_part("feed_forward", "gated_mlp", GatedFeedForward, replace=True)
+register_part("feed_forward", "capped_gated_mlp", CappedGatedFeedForward, replace=True)

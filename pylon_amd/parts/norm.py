@@ -9,7 +9,7 @@ import torch
 
 from ..config.specs import NormSpec
 from ..kernels import ops
-from .base import Part
+from .base import Normed, Part
 from .registry import register_part
 
 
@@ -23,10 +23,40 @@ class RMSNorm(Part):
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return ops.rmsnorm(x, self.params["weight"], self.spec.eps, out_dtype=self.dtype)
 
-    def add_forward(self, resid: torch.Tensor, delta: Optional[torch.Tensor], *,
+    def add_forward(self, resid: torch.Tensor, delta, *,
                     row_idx: Optional[torch.Tensor] = None) -> torch.Tensor:
+        if isinstance(delta, Normed):
+            return ops.add_normed_rmsnorm(resid, delta.value, self.params["weight"], self.spec.eps, self.dtype,
+                                          post_gain=delta.gain, post_eps=delta.eps, row_idx=row_idx)
         return ops.add_rmsnorm(resid, delta, self.params["weight"], self.spec.eps, self.dtype,
                                row_idx=row_idx)
 
 
+class ScalarRMSNorm(Part):
+    """``g * x / sqrt(mean(x^2) + eps)`` with one learned number ``g`` for all coordinates, in
+    float32.  As the norm after a sublayer it is not applied here: :meth:`pending` wraps the
+    sublayer's output with the gain, and the next norm's kernel norms it, adds it to the residual
+    stream and norms the sum in one pass."""
+
+    def __init__(self, spec: NormSpec, *, dtype: torch.dtype, device) -> None:
+        super().__init__()
+        self.spec = spec
+        self.dtype = dtype
+        self.add_param("weight", (), torch.float32, device, role="vector")
+
+    def pending(self, value: torch.Tensor) -> Normed:
+        return Normed(value, self.params["weight"], self.spec.eps)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return ops.add_normed_rmsnorm(x.float() if x.dtype != torch.float32 else x, None, self.params["weight"],
+                                      self.spec.eps, self.dtype)
+
+    def add_forward(self, resid: torch.Tensor, delta, *, row_idx: Optional[torch.Tensor] = None) -> torch.Tensor:
+        if isinstance(delta, Normed):
+            return ops.add_normed_rmsnorm(resid, delta.value, self.params["weight"], self.spec.eps, self.dtype,
+                                          post_gain=delta.gain, post_eps=delta.eps, row_idx=row_idx)
+        return ops.add_normed_rmsnorm(resid, delta, self.params["weight"], self.spec.eps, self.dtype, row_idx=row_idx)
+
+
 register_part("norm", "rmsnorm", RMSNorm, replace=True)
+register_part("norm", "scalar_rmsnorm", ScalarRMSNorm, replace=True)

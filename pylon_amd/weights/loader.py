@@ -57,6 +57,18 @@ def shard_files(folder: Path) -> List[Path]:
     return [folder / "model.safetensors"]
 
 
+def tensor_shapes(folder) -> Dict[str, Tuple[int, ...]]:
+    """``{tensor name: shape}`` of a model folder, from the shards' headers alone."""
+    shapes: Dict[str, Tuple[int, ...]] = {}
+    for path in shard_files(Path(folder)):
+        if not path.is_file():
+            raise FileNotFoundError(f"{path} does not exist")
+        with safe_open(str(path), framework="pt", device="cpu") as f:
+            for name in f.keys():
+                shapes[name] = tuple(f.get_slice(name).get_shape())
+    return shapes
+
+
 def _param_dtype(model_dtype: torch.dtype, role: str, stored: List[str]) -> torch.dtype:
     if role == "table":
         return torch.int32
