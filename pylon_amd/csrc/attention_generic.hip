@@ -1,5 +1,5 @@
 // Paged causal grouped-query attention, the exact and general form: any element type,
-// any head size that is a multiple of 16 (up to 512), any number of heads and groups,
+// any head size up to 512 (multiples of 8 with 16-byte loads), any number of heads and groups,
 // any page size, optional sliding window.  One wavefront owns one (token, query head):
 // it walks that token's visible keys 64 at a time (one key per lane), keeps a running
 // maximum and sum in float, and accumulates the weighted values with one lane per
@@ -91,7 +91,11 @@ __global__ void paged_attention_kernel(T* __restrict__ out, const T* __restrict_
       phys = table[j / page_size] * page_size + (j % page_size);
       const T* kr = k_cache + (static_cast<size_t>(phys) * n_kv_heads + kvh) * head_dim;
       float dot = 0.f;
-      for (int d = 0; d < head_dim; d += 8) dot = Vec8<T>::dot(qbuf + d, kr + d, dot);
+      if (head_dim & 7) {  // a head that is no whole number of 16-byte pieces: element by element
+        for (int d = 0; d < head_dim; ++d) dot = fmaf(qbuf[d], to_float(kr[d]), dot);
+      } else {
+        for (int d = 0; d < head_dim; d += 8) dot = Vec8<T>::dot(qbuf + d, kr + d, dot);
+      }
       s = dot * scale;
       if (rel != nullptr) {
         const int far = pos - j;
@@ -171,8 +175,7 @@ extern "C" int pylon_paged_attention(void* out, const void* q, const void* k_cac
   PYLON_REQUIRE(tokens >= 0 && n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
                 "paged_attention: %d query heads cannot be grouped over %d key/value heads", n_heads,
                 n_kv_heads);
-  PYLON_REQUIRE(head_dim >= 8 && head_dim % 8 == 0 && head_dim <= 512,
-                "paged_attention: head_dim %d must be a multiple of 8 between 8 and 512", head_dim);
+  PYLON_REQUIRE(head_dim >= 1 && head_dim <= 512, "paged_attention: head_dim %d must be between 1 and 512", head_dim);
   PYLON_REQUIRE(page_size > 0 && table_width > 0, "paged_attention: bad page size or table width");
   PYLON_REQUIRE(v_dim >= 1 && v_dim <= 512, "paged_attention: values of 1 to 512 elements, got %d", v_dim);
   PYLON_REQUIRE(q_stride >= static_cast<long long>(n_heads) * head_dim, "paged_attention: q rows overlap");

@@ -155,9 +155,9 @@ class SinkAttention(Part):
         super().__init__()
         if spec.n_heads % spec.n_kv_heads:
             raise ValueError("The number of Q heads must be divisible by the number of KV heads.")
-        if spec.head_dim % 8 or not 8 <= spec.head_dim <= 512 or not 1 <= spec.v_head_dim <= 512:
+        if not 1 <= spec.head_dim <= 512 or not 1 <= spec.v_head_dim <= 512:
             raise ValueError(f"heads of {spec.head_dim} key and {spec.v_head_dim} value elements are not supported: "
-                             "keys take multiples of 8 up to 512, values 1 to 512")
+                             "both take 1 to 512")
         if spec.window is not None and spec.window < 1:
             raise ValueError("window must be positive (or None for full attention)")
         self.spec = spec

@@ -904,10 +904,10 @@ def test_decode_attention_that_prepares_q_k_v_itself(ops, geom, store):
 def test_kernels_refuse_what_they_cannot_do(ops):
     from pylon_amd.kernels import KernelError
 
-    q = torch.zeros((1, 2, 24), device=DEV)
-    kc = torch.zeros((2, 16, 1, 24), device=DEV)
+    q = torch.zeros((1, 2, 520), device=DEV)
+    kc = torch.zeros((2, 16, 1, 520), device=DEV)
     z = torch.zeros(1, dtype=torch.int32, device=DEV)
-    with pytest.raises(KernelError, match="multiple of 16"):
+    with pytest.raises(KernelError, match="between 1 and 512"):
         ops.paged_attention(q, kc, kc, torch.zeros((1, 1), dtype=torch.int32, device=DEV), z, z,
                             page_size=16, window=None, scale=1.0)
     with pytest.raises(KernelError, match="cannot be grouped"):
