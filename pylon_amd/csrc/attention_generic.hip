@@ -55,7 +55,7 @@ __global__ void paged_attention_kernel(T* __restrict__ out, const T* __restrict_
                                        long long items, int n_heads, int n_kv_heads, int head_dim,
                                        int page_size, int window, float scale, int v_dim, long long q_stride,
                                        const float* __restrict__ rel, const int* __restrict__ bucket,
-                                       int bucket_len, int sink) {
+                                       int bucket_len, int sink, int v_transposed) {
   extern __shared__ float lds[];
   const int lane = threadIdx.x & (PYLON_WAVE - 1);
   const int wave = threadIdx.x / PYLON_WAVE;
@@ -112,11 +112,16 @@ __global__ void paged_attention_kernel(T* __restrict__ out, const T* __restrict_
     for (int kk = 0; kk < count; ++kk) {
       const float pk = __shfl(p, kk, PYLON_WAVE);
       const int physk = __shfl(phys, kk, PYLON_WAVE);
-      const T* vr = v_cache + (static_cast<size_t>(physk) * n_kv_heads + kvh) * v_dim;
+      // values transposed inside their page: [page, kv head, element, slot in page]
+      const T* vr = v_transposed
+                        ? v_cache + (static_cast<size_t>(physk / page_size) * n_kv_heads + kvh) * v_dim * page_size +
+                              physk % page_size
+                        : v_cache + (static_cast<size_t>(physk) * n_kv_heads + kvh) * v_dim;
+      const size_t vstep = v_transposed ? page_size : 1;
 #pragma unroll
       for (int i = 0; i < DIMS_PER_LANE; ++i) {
         const int d = lane + PYLON_WAVE * i;
-        if (d < v_dim) acc[i] = fmaf(pk, to_float(vr[d]), acc[i]);
+        if (d < v_dim) acc[i] = fmaf(pk, to_float(vr[d * vstep]), acc[i]);
       }
     }
     m = m_new;
@@ -137,7 +142,7 @@ static int launch_paged_attention(T* out, const T* q, const T* k_cache, const T*
                                   const int* positions, int tokens, int n_heads, int n_kv_heads,
                                   int head_dim, int page_size, int window, float scale, int v_dim,
                                   long long q_stride, const float* rel, const int* bucket, int bucket_len,
-                                  int sink, hipStream_t stream) {
+                                  int sink, int v_transposed, hipStream_t stream) {
   const long long items = static_cast<long long>(tokens) * n_heads;
   const long long blocks = (items + ATT_WAVES - 1) / ATT_WAVES;
   dim3 grid((unsigned)blocks), block(ATT_WAVES * PYLON_WAVE);
@@ -146,7 +151,7 @@ static int launch_paged_attention(T* out, const T* q, const T* k_cache, const T*
   hipLaunchKernelGGL((paged_attention_kernel<T, DPL>), grid, block, lds, stream, out, q, k_cache,    \
                      v_cache, block_table, table_width, tok_row, positions, items, n_heads,          \
                      n_kv_heads, head_dim, page_size, window, scale, v_dim, q_stride, rel, bucket,   \
-                     bucket_len, sink)
+                     bucket_len, sink, v_transposed)
   if (v_dim <= 64)
     LAUNCH(1);
   else if (v_dim <= 128)
@@ -161,6 +166,7 @@ static int launch_paged_attention(T* out, const T* q, const T* k_cache, const T*
 
 // q: [tokens, n_heads, head_dim], rows q_stride elements apart; out: [tokens, n_heads, v_dim].
 // Caches: keys [pages*page_size, n_kv_heads, head_dim], values [pages*page_size, n_kv_heads, v_dim].
+// With v_transposed the values lie as [pages, n_kv_heads, v_dim, page_size].
 // rel: null, or float [rows, n_heads] with bucket: int [bucket_len], every entry a row of rel.
 // block_table: [rows, table_width] page ids; tok_row[t] names the table row of token t;
 // positions[t] is the token's index in its request; keys first(t)..positions[t] are read,
@@ -170,7 +176,8 @@ extern "C" int pylon_paged_attention(void* out, const void* q, const void* k_cac
                                      const int* tok_row, const int* positions, int tokens, int n_heads,
                                      int n_kv_heads, int head_dim, int page_size, int window,
                                      float scale, int v_dim, long long q_stride, const float* rel,
-                                     const int* bucket, int bucket_len, int sink, hipStream_t stream) {
+                                     const int* bucket, int bucket_len, int sink, int v_transposed,
+                                     hipStream_t stream) {
   PYLON_REQUIRE(pylon_valid_dtype(dtype), "paged_attention: unknown dtype");
   PYLON_REQUIRE(tokens >= 0 && n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
                 "paged_attention: %d query heads cannot be grouped over %d key/value heads", n_heads,
@@ -189,11 +196,11 @@ extern "C" int pylon_paged_attention(void* out, const void* q, const void* k_cac
     launch_paged_attention<float>((float*)out, (const float*)q, (const float*)k_cache,
                                   (const float*)v_cache, block_table, table_width, tok_row, positions,
                                   tokens, n_heads, n_kv_heads, head_dim, page_size, window, scale, v_dim,
-                                  q_stride, rel, bucket, bucket_len, sink, stream);
+                                  q_stride, rel, bucket, bucket_len, sink, v_transposed, stream);
   else
     launch_paged_attention<bf16_t>((bf16_t*)out, (const bf16_t*)q, (const bf16_t*)k_cache,
                                    (const bf16_t*)v_cache, block_table, table_width, tok_row, positions,
                                    tokens, n_heads, n_kv_heads, head_dim, page_size, window, scale, v_dim,
-                                   q_stride, rel, bucket, bucket_len, sink, stream);
+                                   q_stride, rel, bucket, bucket_len, sink, v_transposed, stream);
   PYLON_LAUNCHED("paged_attention");
 }

@@ -1,0 +1,271 @@
+// Paged causal attention with a learned bias by distance and a sink, on the matrix cores, for
+// bfloat16 prompt portions and single tokens alike:
+//
+//   s_ij = scale * q_i.k_j + rel[bucket[min(i - j, bucket_len - 1)], head],   j <= i
+//   out_i = sum_j exp(s_ij) v_j / (1 + sum_j exp(s_ij))
+//
+// Keys have `dim` elements, values `vdim`.  Keys lie in the cache as [slot, kv head, dim];
+// values lie transposed inside every page, [page, kv head, vdim, slot in page], so that the
+// eight keys a lane feeds to a matrix instruction are neighbours in memory.
+//
+// A wavefront owns up to 32 consecutive tokens of one request and one query head, as two tiles
+// of 16 query columns.  It walks the keys in blocks of 32 (which never cross a page: pages are
+// multiples of 32).  Scores are computed transposed, S^T = K Q^T (16x16x32 instructions: rows are
+// keys, columns are queries), so that everything that belongs to a query (its running maximum,
+// its sum, its output) lives in the lanes of that query's column, and the exponentials are
+// already laid out as the operand of O^T = V^T P^T.  Scores, bias, maximum, exponentials and
+// sums are float; the weights enter the value product as two bfloat16 terms, p = hi + lo, so
+// that they carry sixteen bits of mantissa.  The sink is where the walk starts: maximum 0,
+// sum 1, output 0.  The waves of a workgroup take heads of one key/value head, so that the keys
+// and values one of them fetched are in the nearest cache for the others.  The order of a
+// query's sums depends on its position only.
+#include "common.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+
+#define AS_BLOCK 32   // keys per step of the walk
+#define AS_QT 2       // query tiles of 16 per wave
+#define AS_MAX_BIAS 4096
+
+__device__ __forceinline__ uint32_t as_pack(float a, float b) {
+  return static_cast<uint32_t>(float_to_bf16_bits(a)) | (static_cast<uint32_t>(float_to_bf16_bits(b)) << 16);
+}
+
+// KS: steps of 32 key elements (dim <= 32 KS); NV: tiles of 16 value elements (vdim <= 16 NV).
+template <int KS, int NV>
+__global__ __launch_bounds__(256) void attention_sink_kernel(
+    bf16_t* __restrict__ out, const bf16_t* __restrict__ q, long long q_stride, const bf16_t* __restrict__ k_cache,
+    const bf16_t* __restrict__ v_cache, const int* __restrict__ block_table, int table_width,
+    const int* __restrict__ tiles, const int* __restrict__ positions, int n_heads, int n_kv_heads, int dim, int vdim, int page_size, float scale,
+    const float* __restrict__ rel, const int* __restrict__ bucket, int bucket_len, int sink, int waves_per_group) {
+  extern __shared__ float bias_lds[];  // [waves][bucket_len]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int col = lane & 15, grp = lane >> 4;
+  const int group = n_heads / n_kv_heads;
+  const int chunks = (group + waves_per_group - 1) / waves_per_group;
+  int b = blockIdx.x;
+  const int chunk = b % chunks;
+  b /= chunks;
+  const int kvh = b % n_kv_heads;
+  const int tile = b / n_kv_heads;
+  const int in_group = chunk * waves_per_group + wave;
+  if (in_group >= group) return;  // no barrier below: a wave may leave alone
+  const int head = kvh * group + in_group;
+  // without a table of tiles every token is a tile of its own and row t of the block table is token t's
+  const int tok0 = tiles ? tiles[4 * tile] : tile, count = tiles ? tiles[4 * tile + 1] : 1;
+  const int row = tiles ? tiles[4 * tile + 2] : tile, pos0 = tiles ? tiles[4 * tile + 3] : positions[tile];
+  const int kv_last = pos0 + count - 1;
+  const int* table = block_table + static_cast<size_t>(row) * table_width;
+
+  float* tbl = bias_lds + wave * bucket_len;
+  if (rel != nullptr)
+    for (int d = lane; d < bucket_len; d += 64) tbl[d] = rel[static_cast<size_t>(bucket[d]) * n_heads + head];
+  const float far_bias = rel != nullptr ? rel[static_cast<size_t>(bucket[bucket_len - 1]) * n_heads + head] : 0.f;
+
+  // Q^T operands: column = query, eight key elements per lane and step
+  bf16x8 qf[AS_QT][KS];
+  int qpos[AS_QT];
+#pragma unroll
+  for (int qt = 0; qt < AS_QT; ++qt) {
+    const int qi = qt * 16 + col;
+    qpos[qt] = pos0 + qi;
+    const int t = tok0 + (qi < count ? qi : count - 1);
+    const bf16_t* qr = q + static_cast<size_t>(t) * q_stride + static_cast<size_t>(head) * dim;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int d = ks * 32 + grp * 8;
+      u32x4 raw = {0u, 0u, 0u, 0u};
+      if (d < dim) raw = *reinterpret_cast<const u32x4*>(qr + d);
+      qf[qt][ks] = __builtin_bit_cast(bf16x8, raw);
+    }
+  }
+
+  floatx4 o[AS_QT][NV];
+  float m_run[AS_QT], l_run[AS_QT];
+#pragma unroll
+  for (int qt = 0; qt < AS_QT; ++qt) {
+    // the sink: a key of score 0 without a value (one lane of a query's four carries its one)
+    m_run[qt] = sink ? 0.f : -INFINITY;
+    l_run[qt] = (sink && grp == 0) ? 1.f : 0.f;
+#pragma unroll
+    for (int dt = 0; dt < NV; ++dt) o[qt][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  for (int kb = 0; kb <= kv_last; kb += AS_BLOCK) {
+    const int page = table[kb / page_size];
+    const int in_page = kb % page_size;
+    // K operands: row = key, eight elements per lane and step
+    floatx4 s[AS_QT][2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const size_t slot = static_cast<size_t>(page) * page_size + in_page + t * 16 + col;
+      const bf16_t* kr = k_cache + (slot * n_kv_heads + kvh) * dim;
+#pragma unroll
+      for (int qt = 0; qt < AS_QT; ++qt) s[qt][t] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const int d = ks * 32 + grp * 8;
+        u32x4 raw = {0u, 0u, 0u, 0u};
+        if (d < dim) raw = *reinterpret_cast<const u32x4*>(kr + d);
+        const bf16x8 kf = __builtin_bit_cast(bf16x8, raw);
+#pragma unroll
+        for (int qt = 0; qt < AS_QT; ++qt)
+          s[qt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[qt][ks], s[qt][t], 0, 0, 0);
+      }
+    }
+    // V^T operands: row = value element, keys kb + 4 grp + {0..3} and kb + 16 + 4 grp + {0..3}
+    bf16x8 vf[NV];
+    const bool ragged = kb + AS_BLOCK - 1 > kv_last;  // slots past the request's end hold anything
+#pragma unroll
+    for (int dt = 0; dt < NV; ++dt) {
+      const int d = dt * 16 + col;
+      u32x4 raw = {0u, 0u, 0u, 0u};
+      if (d < vdim) {
+        const bf16_t* vr = v_cache + ((static_cast<size_t>(page) * n_kv_heads + kvh) * vdim + d) * page_size +
+                           in_page + 4 * grp;
+        const u32x2 first = *reinterpret_cast<const u32x2*>(vr);
+        const u32x2 second = *reinterpret_cast<const u32x2*>(vr + 16);
+        raw = u32x4{first[0], first[1], second[0], second[1]};
+        if (ragged) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const int key = kb + (e >> 2) * 16 + 4 * grp + (e & 3);
+            if (key > kv_last) raw[e >> 1] &= (e & 1) ? 0x0000ffffu : 0xffff0000u;
+          }
+        }
+      }
+      vf[dt] = __builtin_bit_cast(bf16x8, raw);
+    }
+
+#pragma unroll
+    for (int qt = 0; qt < AS_QT; ++qt) {
+      // scores of this lane: keys kb + 16 t + 4 grp + i for query qpos[qt]
+      float sc[8];
+      const int near = qpos[qt] - (kb + AS_BLOCK - 1);  // the smallest distance of the block for this query
+      const bool all_far = rel == nullptr || near >= bucket_len - 1;
+      float top = m_run[qt];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int key = kb + (e >> 2) * 16 + 4 * grp + (e & 3);
+        const int dist = qpos[qt] - key;
+        float bias = far_bias;
+        if (!all_far) {
+          int idx = dist < 0 ? 0 : dist;
+          idx = idx < bucket_len - 1 ? idx : bucket_len - 1;
+          bias = tbl[idx];
+        }
+        const float v = fmaf(s[qt][e >> 2][e & 3], scale, bias);
+        sc[e] = dist >= 0 ? v : -INFINITY;
+        top = fmaxf(top, sc[e]);
+      }
+      top = fmaxf(top, __shfl_xor(top, 16, 64));
+      top = fmaxf(top, __shfl_xor(top, 32, 64));
+      // a query past the tile's end, or one whose every key so far is hidden, keeps -inf: no NaN from inf - inf
+      const float m_new = top;
+      const float corr = (m_new == -INFINITY) ? 1.f : __expf(m_run[qt] - m_new);
+      float p[8], sum = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        p[e] = (sc[e] == -INFINITY) ? 0.f : __expf(sc[e] - m_new);
+        sum += p[e];
+      }
+      l_run[qt] = l_run[qt] * corr + sum;
+      m_run[qt] = m_new;
+      u32x4 hi, lo;
+#pragma unroll
+      for (int e = 0; e < 8; e += 2) {
+        const uint32_t h = as_pack(p[e], p[e + 1]);
+        hi[e >> 1] = h;
+        lo[e >> 1] = as_pack(p[e] - __uint_as_float(h << 16), p[e + 1] - __uint_as_float(h & 0xffff0000u));
+      }
+      const bf16x8 p_hi = __builtin_bit_cast(bf16x8, hi), p_lo = __builtin_bit_cast(bf16x8, lo);
+#pragma unroll
+      for (int dt = 0; dt < NV; ++dt) {
+        floatx4 acc = o[qt][dt];
+        acc[0] *= corr; acc[1] *= corr; acc[2] *= corr; acc[3] *= corr;
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], p_hi, acc, 0, 0, 0);
+        o[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], p_lo, acc, 0, 0, 0);
+      }
+    }
+  }
+
+#pragma unroll
+  for (int qt = 0; qt < AS_QT; ++qt) {
+    float l = l_run[qt];
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+    const int qi = qt * 16 + col;
+    if (qi >= count) continue;
+    const float inv = 1.0f / l;
+    bf16_t* orow = out + (static_cast<size_t>(tok0 + qi) * n_heads + head) * vdim;
+#pragma unroll
+    for (int dt = 0; dt < NV; ++dt) {
+      const int d = dt * 16 + 4 * grp;
+      if (d + 3 < vdim) {
+        u32x2 packed = {as_pack(o[qt][dt][0] * inv, o[qt][dt][1] * inv), as_pack(o[qt][dt][2] * inv, o[qt][dt][3] * inv)};
+        *reinterpret_cast<u32x2*>(orow + d) = packed;
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (d + i < vdim) orow[d + i].bits = float_to_bf16_bits(o[qt][dt][i] * inv);
+      }
+    }
+  }
+}
+
+// q: bf16 [tokens, n_heads, dim], rows q_stride elements apart; out: bf16 [tokens, n_heads, vdim].
+// k_cache: bf16 [pages * page_size, n_kv_heads, dim]; v_cache: bf16 [pages, n_kv_heads, vdim, page_size].
+// tiles: int [n_tiles, 4] = (first token, count <= 32, block-table row, first position) of runs of
+// consecutive tokens of one request; or null, and then positions: int [n_tiles], one token per tile,
+// token t on row t of the block table (a step of single tokens).  rel: null or float [rows, n_heads] with bucket: int
+// [bucket_len <= 4096] rows of rel by distance.  dim a multiple of 8 up to 256, vdim a multiple of 4
+// up to 256, page_size a multiple of 32.  The host guarantees that the tiles lie inside q and the table.
+extern "C" int pylon_attention_sink(void* out, const void* q, long long q_stride, const void* k_cache,
+                                    const void* v_cache, const int* block_table, int table_width, const int* tiles,
+                                    const int* positions, int n_tiles, int n_heads, int n_kv_heads, int dim, int vdim, int page_size,
+                                    float scale, const float* rel, const int* bucket, int bucket_len, int sink,
+                                    hipStream_t stream) {
+  PYLON_REQUIRE(n_tiles >= 0 && n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
+                "attention_sink: %d query heads cannot be grouped over %d key/value heads", n_heads, n_kv_heads);
+  PYLON_REQUIRE(dim >= 8 && dim % 8 == 0 && dim <= 256, "attention_sink: keys of a multiple of 8 up to 256 elements, got %d", dim);
+  PYLON_REQUIRE(vdim >= 4 && vdim % 4 == 0 && vdim <= 256, "attention_sink: values of a multiple of 4 up to 256 elements, got %d", vdim);
+  PYLON_REQUIRE(page_size > 0 && page_size % AS_BLOCK == 0, "attention_sink: pages of a multiple of %d tokens, got %d", AS_BLOCK, page_size);
+  PYLON_REQUIRE(table_width > 0 && q_stride >= static_cast<long long>(n_heads) * dim && q_stride % 8 == 0,
+                "attention_sink: bad table width or q stride");
+  PYLON_REQUIRE((reinterpret_cast<uintptr_t>(q) & 15) == 0 && (reinterpret_cast<uintptr_t>(k_cache) & 15) == 0 &&
+                (reinterpret_cast<uintptr_t>(v_cache) & 7) == 0 && (reinterpret_cast<uintptr_t>(out) & 7) == 0,
+                "attention_sink: operands must be 16-byte aligned");
+  PYLON_REQUIRE(tiles != nullptr || positions != nullptr, "attention_sink: tiles or positions are required");
+  PYLON_REQUIRE(rel == nullptr || (bucket != nullptr && bucket_len >= 1 && bucket_len <= AS_MAX_BIAS),
+                "attention_sink: a bias by distance needs a table of 1 to %d buckets", AS_MAX_BIAS);
+  if (n_tiles == 0) return 0;
+  const int group = n_heads / n_kv_heads;
+  const int waves = group < 4 ? group : 4;
+  const int chunks = (group + waves - 1) / waves;
+  const long long blocks = static_cast<long long>(n_tiles) * n_kv_heads * chunks;
+  PYLON_REQUIRE(blocks < (1ll << 31), "attention_sink: too many tiles for one launch");
+  dim3 grid(static_cast<unsigned>(blocks)), block(64 * waves);
+  const size_t lds = rel != nullptr ? sizeof(float) * waves * bucket_len : 0;
+  const int ks = (dim + 31) / 32, nv = (vdim + 15) / 16;
+#define GO(KS, NV)                                                                                                 \
+  hipLaunchKernelGGL((attention_sink_kernel<KS, NV>), grid, block, lds, stream, (bf16_t*)out, (const bf16_t*)q,     \
+                     q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, table_width, tiles,      \
+                     positions, n_heads, n_kv_heads, dim, vdim, page_size, scale, rel, bucket, rel ? bucket_len : 1, sink, waves)
+#define PICK_NV(KS)                 \
+  do {                              \
+    if (nv <= 2) GO(KS, 2);         \
+    else if (nv <= 4) GO(KS, 4);    \
+    else if (nv <= 8) GO(KS, 8);    \
+    else GO(KS, 16);                \
+  } while (0)
+  if (ks <= 1) PICK_NV(1);
+  else if (ks <= 2) PICK_NV(2);
+  else if (ks <= 4) PICK_NV(4);
+  else PICK_NV(8);
+#undef PICK_NV
+#undef GO
+  PYLON_LAUNCHED("attention_sink");
+}

@@ -189,19 +189,25 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                     block_table: torch.Tensor, tok_row: torch.Tensor, positions: torch.Tensor, *,
                     page_size: int, window: Optional[int], scale: float,
                     out: Optional[torch.Tensor] = None, rel: Optional[torch.Tensor] = None,
-                    bucket: Optional[torch.Tensor] = None, sink: bool = False) -> torch.Tensor:
+                    bucket: Optional[torch.Tensor] = None, sink: bool = False,
+                    v_transposed: bool = False) -> torch.Tensor:
     """Causal attention of each token over its request's cached keys ``<=`` its position.
     ``q`` is ``[tokens, heads, head_dim]`` and may be a slice of wider rows (a fused
     projection); values may have another size than keys.  ``rel`` (float32 ``[rows, heads]``)
     with ``bucket`` (int32 ``[n]``) adds ``rel[bucket[min(i - j, n - 1)], head]`` to the scaled
-    score of query ``i`` and key ``j``; ``sink`` adds one to the softmax's denominator."""
+    score of query ``i`` and key ``j``; ``sink`` adds one to the softmax's denominator.  With
+    ``v_transposed`` the values lie as ``[pages, kv_heads, v_dim, page_size]``."""
     if q.dim() != 3:
         raise KernelError("paged_attention takes q as [tokens, heads, head_dim]")
     tokens, n_heads, head_dim = q.shape
-    if k_cache.dim() != 4 or v_cache.dim() != 4 or k_cache.shape[:3] != v_cache.shape[:3]:
+    if v_transposed and v_cache.dim() == 4:
+        v_shape = (v_cache.shape[0], v_cache.shape[3], v_cache.shape[1], v_cache.shape[2])
+    else:
+        v_shape = tuple(v_cache.shape)
+    if k_cache.dim() != 4 or v_cache.dim() != 4 or tuple(k_cache.shape[:3]) != v_shape[:3]:
         raise KernelError("paged_attention: caches must be [pages, page_size, kv_heads, head_dim]")
     pages, psize, n_kv_heads, hd = k_cache.shape
-    v_dim = v_cache.shape[3]
+    v_dim = v_shape[3]
     if q.stride(2) != 1 or q.stride(1) != head_dim or (tokens > 1 and q.stride(0) < n_heads * head_dim):
         raise KernelError("paged_attention: the heads of a q row must lie side by side")
     if (rel is None) != (bucket is None):
@@ -230,7 +236,61 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
               _dev(positions, "positions", torch.int32), tokens, n_heads, n_kv_heads, head_dim,
               page_size, int(window or 0), float(scale), v_dim, q.stride(0) if tokens > 1 else n_heads * head_dim,
               _dev(rel, "rel", torch.float32), _dev(bucket, "bucket", torch.int32),
-              0 if bucket is None else bucket.numel(), 1 if sink else 0, _stream())
+              0 if bucket is None else bucket.numel(), 1 if sink else 0, 1 if v_transposed else 0, _stream())
+    return out
+
+
+SINK_MAX_BIAS = 4096  # distances the matrix-core sink attention keeps a bias for in LDS
+SINK_TILE = 32        # most tokens of one tile of it
+
+
+def attention_sink_ok(dtype: torch.dtype, *, head_dim: int, v_dim: int, page_size: int, bucket_len: int,
+                      window: Optional[int] = None) -> bool:
+    """Whether the matrix-core kernel takes this geometry (else the general kernel does)."""
+    return (dtype == torch.bfloat16 and head_dim % 8 == 0 and 8 <= head_dim <= 256 and v_dim % 4 == 0
+            and 4 <= v_dim <= 256 and page_size % 32 == 0 and bucket_len <= SINK_MAX_BIAS and window is None)
+
+
+def attention_sink(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
+                   tiles: Optional[torch.Tensor], positions: Optional[torch.Tensor], *, page_size: int, scale: float,
+                   rel: Optional[torch.Tensor], bucket: Optional[torch.Tensor], sink: bool) -> torch.Tensor:
+    """Causal attention with a bias by distance and a sink on the matrix cores: bfloat16 ``q``
+    ``[tokens, heads, head_dim]`` (maybe a slice of wider rows), keys ``[pages, page_size, kv_heads,
+    head_dim]``, values transposed inside their pages ``[pages, kv_heads, v_dim, page_size]``.
+    ``tiles`` int32 ``[n, 4]`` (first token, count <= 32, block-table row, first position); or None
+    with ``positions``: every token a tile of its own on its own row of the table."""
+    if q.dim() != 3 or k_cache.dim() != 4 or v_cache.dim() != 4:
+        raise KernelError("attention_sink takes q [tokens, heads, head_dim] and 4-D caches")
+    tokens, n_heads, head_dim = q.shape
+    pages, psize, n_kv_heads, hd = k_cache.shape
+    v_dim = v_cache.shape[2]
+    if v_cache.shape != (pages, n_kv_heads, v_dim, psize) or psize != page_size or hd != head_dim:
+        raise KernelError("attention_sink: cache geometry does not match page_size/head_dim")
+    if not attention_sink_ok(q.dtype, head_dim=head_dim, v_dim=v_dim, page_size=page_size,
+                             bucket_len=0 if bucket is None else bucket.numel()):
+        raise KernelError("attention_sink does not take this geometry")
+    if k_cache.dtype != q.dtype or v_cache.dtype != q.dtype or n_heads % n_kv_heads:
+        raise KernelError("attention_sink: q and the caches differ in dtype, or the heads do not group")
+    if q.stride(2) != 1 or q.stride(1) != head_dim or (tokens > 1 and q.stride(0) < n_heads * head_dim):
+        raise KernelError("attention_sink: the heads of a q row must lie side by side")
+    if pages * page_size >= 2 ** 31 or block_table.dim() != 2:
+        raise KernelError("attention_sink: the cache is too large for int32 slots, or the table is not 2-D")
+    if (rel is None) != (bucket is None) or (rel is not None and (rel.dim() != 2 or rel.shape[1] != n_heads)):
+        raise KernelError("attention_sink: rel [rows, heads] and bucket go together")
+    if tiles is not None:
+        if tiles.dim() != 2 or tiles.shape[1] != 4:
+            raise KernelError("attention_sink: tiles must be [n, 4]")
+        n_tiles = tiles.shape[0]
+    else:
+        if positions is None or positions.numel() != tokens or block_table.shape[0] < tokens:
+            raise KernelError("attention_sink: without tiles, one position and one table row per token")
+        n_tiles = tokens
+    out = torch.empty((tokens, n_heads, v_dim), dtype=q.dtype, device=q.device)
+    _lib.call("pylon_attention_sink", _dev(out, "out"), q.data_ptr(), q.stride(0) if tokens > 1 else n_heads * head_dim,
+              _dev(k_cache, "k_cache"), _dev(v_cache, "v_cache"), _dev(block_table, "block_table", torch.int32),
+              block_table.shape[1], _dev(tiles, "tiles", torch.int32), _dev(positions, "positions", torch.int32),
+              n_tiles, n_heads, n_kv_heads, head_dim, v_dim, page_size, float(scale), _dev(rel, "rel", torch.float32),
+              _dev(bucket, "bucket", torch.int32), 0 if bucket is None else bucket.numel(), 1 if sink else 0, _stream())
     return out
 
 
@@ -326,9 +386,10 @@ def retention_recurrent(proj: torch.Tensor, state: torch.Tensor, decay: torch.Te
 
 
 def kv_store(proj: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, slot_map: torch.Tensor, *,
-             k_off: int, v_off: int) -> None:
+             k_off: int, v_off: int, v_transposed: bool = False) -> None:
     """Copy every token's keys (``proj[t, k_off:]``) and values (``proj[t, v_off:]``) into its
-    cache slot; the caches are ``[pages, page_size, kv_heads, size]`` with sizes of their own."""
+    cache slot; the caches are ``[pages, page_size, kv_heads, size]`` with sizes of their own.
+    With ``v_transposed`` the values go to ``[pages, kv_heads, size, page_size]``."""
     if proj.dim() != 2 or proj.stride(1) != 1 or k_cache.dim() != 4 or v_cache.dim() != 4:
         raise KernelError("kv_store takes a 2-D projection and 4-D caches")
     if k_cache.dtype != proj.dtype or v_cache.dtype != proj.dtype:
@@ -336,14 +397,18 @@ def kv_store(proj: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, s
     tokens = proj.shape[0]
     if slot_map.numel() != tokens:
         raise KernelError("kv_store: one cache slot per token is required")
-    k_row, v_row = k_cache.shape[2] * k_cache.shape[3], v_cache.shape[2] * v_cache.shape[3]
+    k_row = k_cache.shape[2] * k_cache.shape[3]
+    v_row = v_cache.shape[1] * v_cache.shape[2] if v_transposed else v_cache.shape[2] * v_cache.shape[3]
+    page_size = k_cache.shape[1]
+    if v_cache.numel() != k_cache.shape[0] * page_size * v_row:
+        raise KernelError("kv_store: the two caches hold different numbers of slots")
     if max(k_off + k_row, v_off + v_row) > proj.shape[1]:
         raise KernelError("kv_store: keys or values lie outside the projection's rows")
     if not proj.is_cuda:
         raise KernelError("proj must live on the GPU; there is no CPU path")
     _lib.call("pylon_kv_store", _dev(k_cache, "k_cache"), _dev(v_cache, "v_cache"), proj.data_ptr(),
               dtype_code(proj.dtype), proj.stride(0), int(k_off), int(v_off), _dev(slot_map, "slot_map", torch.int32),
-              tokens, k_row, v_row, _stream())
+              tokens, k_row, v_row, page_size if v_transposed else 0, _stream())
 
 
 def gated_act(gate_up: torch.Tensor, *, alpha: float, offset: float, limit: float,

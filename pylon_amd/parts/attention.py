@@ -148,8 +148,11 @@ def distance_buckets(rows: int, far: float) -> list:
 class SinkAttention(Part):
     """Grouped-query attention over the paged cache with a learned bias by distance in place
     of a rotation, a sink in the softmax's denominator, and values of another size than keys.
-    ``[q; k; v] = W h`` in one product; k and v go to the tokens' cache slots as they are;
-    scores, bias and softmax are float32."""
+    ``[q; k; v] = W h`` in one product; k and v go to the tokens' cache slots as they are, the
+    values transposed inside their page (slot in page fastest), which is how the matrix-core
+    kernel reads them; scores, bias and softmax are float32.  bfloat16 steps over pages of a
+    multiple of 32 tokens run on the matrix cores (prompt portions as tiles of up to 32 tokens,
+    a step of single tokens as one tile a token); everything else on the general kernel."""
 
     def __init__(self, spec: SinkAttentionSpec, *, dtype: torch.dtype, device) -> None:
         super().__init__()
@@ -182,12 +185,23 @@ class SinkAttention(Part):
         tokens = h.shape[0]
         weight = self.params["qkv"] if stores else self.params["qkv"][: self.q_size]
         qkv = ops.linear(h, weight, out_dtype=self.dtype)
+        pages, page_size = cache.v.shape[0], cache.page_size
+        v_cache = cache.v.view(pages, spec.n_kv_heads, spec.v_head_dim, page_size)
         if stores:
-            ops.kv_store(qkv, cache.k, cache.v, cache.slot_map, k_off=self.q_size, v_off=self.q_size + self.k_size)
-        q = qkv[:, : self.q_size].view(tokens, spec.n_heads, spec.head_dim)
-        context = ops.paged_attention(
-            q, cache.k, cache.v, cache.block_table, ctx.tok_row, ctx.positions, page_size=cache.page_size,
-            window=spec.window, scale=spec.scale, rel=self.params["rel"], bucket=self.bucket, sink=spec.sink)
+            ops.kv_store(qkv, cache.k, v_cache, cache.slot_map, k_off=self.q_size, v_off=self.q_size + self.k_size,
+                         v_transposed=True)
+        q = qkv.as_strided((tokens, spec.n_heads, spec.head_dim), (qkv.stride(0), spec.head_dim, 1))
+        if ops.attention_sink_ok(self.dtype, head_dim=spec.head_dim, v_dim=spec.v_head_dim, page_size=page_size,
+                                 bucket_len=self.bucket.numel(), window=spec.window) and qkv.stride(0) % 8 == 0:
+            tiles = None if ctx.decode_only else ctx.token_tiles(ops.SINK_TILE)
+            context = ops.attention_sink(q, cache.k, v_cache, cache.block_table, tiles, ctx.positions,
+                                         page_size=page_size, scale=spec.scale, rel=self.params["rel"],
+                                         bucket=self.bucket, sink=spec.sink)
+        else:
+            context = ops.paged_attention(
+                q, cache.k, v_cache, cache.block_table, ctx.tok_row, ctx.positions, page_size=page_size,
+                window=spec.window, scale=spec.scale, rel=self.params["rel"], bucket=self.bucket, sink=spec.sink,
+                v_transposed=True)
         return ops.linear_for_residual(context.view(tokens, spec.n_heads * spec.v_head_dim), self.params["out"],
                                        out_dtype=self.dtype)
 

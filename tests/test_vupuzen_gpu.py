@@ -198,6 +198,60 @@ def test_sink_attention_kernel_sees_far_keys_bucket_edges_and_the_sink(ops, dtyp
     assert np.abs(no_sink - got).max() > 0.01
 
 
+@pytest.mark.parametrize("dim, vdim, heads, groups, rows, far, page", [
+    (64, 64, 4, 1, 16, 300, 32), (96, 48, 6, 3, 32, 130, 64), (16, 24, 4, 2, 12, 20, 32), (40, 12, 3, 3, 6, 9.5, 96),
+    (128, 128, 8, 1, 32, 70, 64), (8, 4, 2, 1, 4, 3, 32)])
+def test_sink_attention_on_the_matrix_cores(ops, dim, vdim, heads, groups, rows, far, page):
+    """The bfloat16 kernel against the plain rule: a prompt portion behind cached tokens, cut into
+    tiles in the order the step function gives them, and single tokens of requests of unequal
+    lengths.  Free slots of the last page hold NaN."""
+    from pylon_amd.parts.attention import distance_buckets
+
+    rng = np.random.default_rng(dim * 7 + vdim)
+    rnd = lambda a: torch.tensor(a).to(torch.bfloat16).to(torch.float64).numpy()
+    total = 333
+    q, k, v = rnd(rng.normal(size=(total, heads, dim))), rnd(rng.normal(size=(total, groups, dim))), rnd(rng.normal(size=(total, groups, vdim)))
+    k[3] *= 5.0
+    q[-5:, 0] = rnd(k[3, 0] * 0.9)  # a far key carries the last queries of head 0
+    k[page] *= 4.0
+    q[200:210, heads - 1] = rnd(k[page, groups - 1] * 1.3)  # a key on a page's first slot
+    q[250:270] *= 0.0  # the biases alone decide there
+    rel = rnd(rng.normal(size=(rows, heads)) * 3.0 - 4.0)
+    scale = 0.17
+    want = plain.sink_softmax_attention(q.transpose(1, 0, 2), k.transpose(1, 0, 2), v.transpose(1, 0, 2), rel, scale, far)
+    want = want.transpose(1, 0, 2)
+    n_pages = 30
+    order = rng.permutation(n_pages)[: math.ceil(total / page)]
+    kc = torch.tensor(paged(k, page, order, n_pages), dtype=torch.bfloat16, device=DEV)  # NaN where no token lies
+    vc = torch.tensor(paged(v, page, order, n_pages), dtype=torch.bfloat16, device=DEV)
+    vt = vc.permute(0, 2, 3, 1).contiguous()  # [pages, kv heads, vdim, slot in page]
+    table = torch.zeros((3, 16), dtype=torch.int32, device=DEV)
+    table[1, : len(order)] = i32(order)
+    bucket, rel_t = i32(distance_buckets(rows, far)), torch.tensor(rel, dtype=torch.float32, device=DEV)
+    first = 140
+    count = total - first
+    wide = torch.zeros((count, heads * dim + 24), dtype=torch.bfloat16, device=DEV)
+    wide[:, : heads * dim] = torch.tensor(q[first:].reshape(count, -1), dtype=torch.bfloat16)
+    qv = wide.as_strided((count, heads, dim), (wide.stride(0), dim, 1))
+    tiles = [(a, min(32, count - a), 1, first + a) for a in range(0, count, 32)]
+    tiles = i32(np.array(tiles[::-1]).reshape(-1)).view(-1, 4)  # heaviest first, as the step function orders them
+    common = dict(page_size=page, scale=scale, rel=rel_t, bucket=bucket, sink=True)
+    got = ops.attention_sink(qv, kc, vt, table, tiles, None, **common).float().cpu().numpy()
+    assert not np.isnan(got).any()
+    assert np.abs(got - want[first:]).max() < 2e-2 * max(1.0, np.abs(want).max())
+    assert np.abs(got[-1, 0] - v[3, 0]).max() < 0.2
+    general = ops.paged_attention(qv, kc.nan_to_num(0.0), vt.nan_to_num(0.0), table, i32([1] * count), i32(range(first, total)),
+                                  window=None, v_transposed=True, **common).float().cpu().numpy()
+    assert np.abs(got - general).max() < 2e-2 * max(1.0, np.abs(want).max())
+    # single tokens: three "requests" that are this sequence at three lengths, one row of the table each
+    lengths = [total, 33, 1]
+    table[0], table[2] = table[1], table[1]
+    singles = torch.tensor(np.stack([q[n - 1] for n in lengths]), dtype=torch.bfloat16, device=DEV)
+    got = ops.attention_sink(singles, kc, vt, table, None, i32([n - 1 for n in lengths]), **common).float().cpu().numpy()
+    for r, n in enumerate(lengths):
+        assert np.abs(got[r] - want[n - 1]).max() < 2e-2 * max(1.0, np.abs(want).max()), n
+
+
 def test_a_sink_takes_all_the_weight_when_every_score_is_far_below_zero(ops):
     rel = torch.full((4, 1), -30.0, device=DEV)
     kc = torch.zeros((1, 16, 1, 8), device=DEV)
@@ -260,11 +314,13 @@ def run_plan(runner, case, plan):
     return {rid: np.concatenate(parts) for rid, parts in got.items() if parts}, pos
 
 
-@pytest.mark.parametrize("name, dtype", [("P", "float32"), ("Q", "float32"), ("R", "float32"), ("R", "bfloat16"),
-                                          ("P", "bfloat16")])
-def test_whole_token_by_token_and_in_portions(tmp, name, dtype):
+@pytest.mark.parametrize("name, dtype, page", [("P", "float32", 16), ("Q", "float32", 16), ("R", "float32", 16),
+                                                ("R", "bfloat16", 16), ("P", "bfloat16", 16), ("R", "bfloat16", 32),
+                                                ("P", "bfloat16", 64), ("Q", "bfloat16", 32)])
+def test_whole_token_by_token_and_in_portions(tmp, name, dtype, page):
+    """Pages of 16 tokens run the general attention kernel, pages of 32 and 64 the matrix-core one."""
     case = Case(tmp, name, dtype, (71, 38))
-    runner = case.runner()
+    runner = case.runner(page_size=page, num_pages=640 // page)
     whole, _ = run_plan(runner, case, [{"r0": 71}, {"r0": 0, "r1": 38}])
     for rid, got in whole.items():
         case.check(rid, got, "whole")
@@ -277,10 +333,12 @@ def test_whole_token_by_token_and_in_portions(tmp, name, dtype):
         assert np.abs(single["r1"] - whole["r1"]).max() <= 2e-5 * np.abs(whole["r1"]).max()
 
 
-@pytest.mark.parametrize("name, dtype", [("P", "float32"), ("Q", "float32"), ("R", "bfloat16")])
-def test_mixed_batches_over_pages_and_slots_that_are_used_again(tmp, name, dtype):
+@pytest.mark.parametrize("name, dtype, page", [("P", "float32", 16), ("Q", "float32", 16), ("R", "bfloat16", 16),
+                                                ("R", "bfloat16", 32), ("P", "bfloat16", 32)])
+def test_mixed_batches_over_pages_and_slots_that_are_used_again(tmp, name, dtype, page):
     case = Case(tmp, name, dtype, (60, 45, 33, 20))
-    runner = case.runner(page_size=16, num_pages=9, max_requests=3)  # room for 144 tokens: never all four at once
+    pages = 9 if page == 16 else 6  # room for 144 (or 192) tokens: never all four requests at once
+    runner = case.runner(page_size=page, num_pages=pages, max_requests=3)
     plan = [{"r0": 20}, {"r0": 1, "r1": 30}, {"r0": 2, "r1": 1, "r2": 5}, {"r0": 1, "r1": 1, "r2": 1},
             {"r0": 20, "r1": 13, "r2": 2}, {"r1": 0, "r0": 1, "r2": 1}, {"r3": 17, "r0": 15, "r2": 24},
             {"r2": 0, "r0": 0, "r3": 1}, {"r3": 2}]
@@ -291,7 +349,7 @@ def test_mixed_batches_over_pages_and_slots_that_are_used_again(tmp, name, dtype
     alone, _ = run_plan(runner, case, [{"r3": 20}])
     limit = 2e-5 if dtype == "float32" else 3e-2
     assert np.abs(alone["r3"] - got["r3"]).max() <= limit * np.abs(alone["r3"]).max()
-    assert runner.manager.free_pages == 9 and runner.manager.slots.free_slots == 3
+    assert runner.manager.free_pages == pages and runner.manager.slots.free_slots == 3
 
 
 def test_long_decoding_after_a_prompt(tmp):
@@ -315,15 +373,16 @@ def test_requests_do_not_see_what_a_freed_slot_or_page_held(tmp):
     assert np.abs(used["r0"] - fresh["r0"]).max() <= 2e-5 * np.abs(fresh["r0"]).max()
 
 
-@pytest.mark.parametrize("name, dtype, graphs", [("P", "float32", False), ("Q", "float32", True), ("R", "bfloat16", True)])
-def test_greedy_generation_through_the_engine(tmp, name, dtype, graphs):
+@pytest.mark.parametrize("name, dtype, graphs, page", [("P", "float32", False, 16), ("Q", "float32", True, 16),
+                                                         ("R", "bfloat16", True, 16), ("R", "bfloat16", True, 32)])
+def test_greedy_generation_through_the_engine(tmp, name, dtype, graphs, page):
     from pylon_amd.engine.engine import Engine
     from pylon_amd.sampling import Sampling
 
     folder = make_folder(tmp, name, dtype=dtype, seed=8)
     cfg, weights = read_folder(folder)
     prompts = [tokens(cfg["vocab"], n, 70 + n) for n in (3, 19, 41)]
-    engine = Engine.from_folder(folder, dtype=dtype, page_size=16, num_pages=24, max_batch_size=3,
+    engine = Engine.from_folder(folder, dtype=dtype, page_size=page, num_pages=384 // page, max_batch_size=3,
                                 prefill_chunk_size=16, cuda_graphs=graphs)
     try:
         results = engine.generate(prompts, Sampling(max_new_tokens=12, temperature=0.0))
