@@ -2,7 +2,7 @@
 and uniform-random token ids, on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L]
-                    [--shape 4b|8b|32b] [--prompt-len N]
+                    [--shape 4b|8b|32b] [--prompt-len N] [--design vupuzen [--design-shapes 8b,...]]
 
 Everything goes the product's own way.  Start-up is ``Runner.from_random``: the fit check,
 the measured activation headroom, the page pool sized from the card's memory and the decode
@@ -288,6 +288,112 @@ def measured_peaks() -> dict:
     return {"hbm_read_gbs": round(read / 1e9, 1), "bf16_gemm_tflops": round(flops / 1e12, 1)}
 
 
+def vupuzen_json(shape: dict, layers: int) -> dict:
+    """A Vupuzen configuration of the shape's layer sizes: every fourth layer retention (as many
+    heads of the shape's head size as fill half the width, so that its four projections together
+    are as large as the attention's), the others attention with the shape's heads and equal key
+    and value sizes; the shape's feed-forward width and vocabulary."""
+    width, hd = shape["hidden_size"], shape["head_dim"]
+    attention = {"type": "attention", "mixer": {
+        "heads": shape["num_attention_heads"], "kv_heads": shape["num_key_value_heads"], "dim": hd, "vdim": hd,
+        "scale": hd ** -0.5, "bias_max": 2048}, "mlp": {"kind": "dense", "ff": shape["intermediate_size"], "limit": 7.0}}
+    heads = max(1, width // (2 * hd))
+    decay = [1.0 - 2.0 ** (-5 - 3 * h / max(1, heads - 1)) for h in range(heads)]
+    retention = {"type": "retention", "mixer": {"heads": heads, "dim": hd, "vdim": hd, "decay": decay,
+                                                "rot": {"dims": hd, "base": 1000000.0}},
+                 "mlp": {"kind": "dense", "ff": shape["intermediate_size"], "limit": 7.0}}
+    return {"architecture": "Vupuzen", "vocab": shape["vocab_size"], "width": width, "canon": {"taps": 4},
+            "norm": {"eps": 1e-6}, "logit_scale": 1.0,
+            "layers": [retention if i % 4 == 0 else attention for i in range(layers)]}
+
+
+def design_steps(runner, vocab: int, batch: int, prompt_len: int, steps: int, warmup: int, seed: int) -> dict:
+    """Milliseconds of one prompt step of ``prompt_len`` tokens (median of five), and of a
+    decode step of ``batch`` requests behind such prompts (mean of ``steps``), through the step
+    function itself: no sampling, the same for every design."""
+    import numpy as np
+    import torch
+
+    from pylon_amd.engine import StepEntry
+
+    rng = np.random.default_rng(seed)
+    times = []
+    for _ in range(6):
+        seq = runner.open(("prompt", len(times)))
+        prompt = rng.integers(0, vocab, prompt_len).tolist()
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        runner.step([StepEntry(seq, prompt, [prompt_len - 1])])
+        end.record()
+        end.synchronize()
+        times.append(start.elapsed_time(end))
+        runner.close(seq)
+    prefill_ms = sorted(times[1:])[2]
+    seqs = [runner.open(("decode", i)) for i in range(batch)]
+    for seq in seqs:
+        runner.step([StepEntry(seq, rng.integers(0, vocab, prompt_len).tolist(), [])])
+    token = [int(t) for t in rng.integers(0, vocab, batch)]
+    for _ in range(warmup):
+        runner.step([StepEntry(seq, [token[i]], [0]) for i, seq in enumerate(seqs)])
+    torch.cuda.synchronize()
+    started = time.perf_counter()
+    for _ in range(steps):
+        runner.step([StepEntry(seq, [token[i]], [0]) for i, seq in enumerate(seqs)])
+    torch.cuda.synchronize()
+    decode_ms = 1e3 * (time.perf_counter() - started) / steps
+    for seq in seqs:
+        runner.close(seq)
+    return {"prefill_ms": round(prefill_ms, 3), "prefill_tokens_per_s": round(1e3 * prompt_len / prefill_ms, 1),
+            "decode_ms": round(decode_ms, 4), "decode_tokens_per_s": round(1e3 * batch / decode_ms, 1)}
+
+
+def design_main(args) -> int:
+    """``--design vupuzen``: prefill and decode of Vupuzen models of random weights at the layer
+    sizes of ``--shape`` (and of the other shapes named by ``--design-shapes``), beside the
+    Qwen3 model of the same sizes and number of layers, both through the same step function
+    over pages of 256 tokens with decode graphs."""
+    import torch
+
+    from pylon_amd.config import PylonConfig
+    from pylon_amd.engine import Runner
+
+    record = None
+    points = {}
+    prompt_len = args.prompt_len if args.prompt_len != PROMPT_LEN else PREFILL_TOKENS
+    steps, warmup = min(args.steps, 128), min(args.warmup, 16)
+    for name in [args.shape] + [n for n in (args.design_shapes or "").split(",") if n and n != args.shape]:
+        shape = SHAPES[name]
+        layers = args.layers or 8
+        pages = (args.batch + 1) * (-(-(prompt_len + steps + warmup + 8) // PAGE_SIZE) + 1)
+        for design, raw in (("vupuzen", vupuzen_json(shape, layers)), ("qwen3", config_json(shape, layers))):
+            config = PylonConfig(dtype=args.dtype, max_batch_size=args.batch + 1, max_queue_size=args.batch + 1,
+                                 page_size=PAGE_SIZE, prefill_chunk_size=prompt_len, num_pages=pages,
+                                 cuda_graphs=not args.no_graphs)
+            runner = Runner.from_random(raw, 0, config, std=0.02)
+            point = design_steps(runner, shape["vocab_size"], args.batch, prompt_len, steps, warmup, seed=3)
+            point["weight_bytes"] = weight_bytes(runner)
+            points[f"{design}_{name}"] = point
+            del runner
+            torch.cuda.empty_cache()
+        mine, theirs = points[f"vupuzen_{name}"], points[f"qwen3_{name}"]
+        points[f"ratio_{name}"] = {"prefill": round(mine["prefill_tokens_per_s"] / theirs["prefill_tokens_per_s"], 3),
+                                   "decode": round(mine["decode_tokens_per_s"] / theirs["decode_tokens_per_s"], 3)}
+        if record is None:
+            record = {
+                "metric": f"decode tokens/s, Vupuzen at the Qwen3-{name.upper()} layer sizes, {layers} layers, "
+                          f"batch {args.batch}, {prompt_len}-token prompts",
+                "value": mine["decode_tokens_per_s"], "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+                "ms_per_step": mine["decode_ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+                "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
+                "config": {"model": f"vupuzen-{name}-sizes-random", "layers": layers, "global_batch": args.batch,
+                           "seq_len": prompt_len, "page_size": PAGE_SIZE, "hip_graphs": not args.no_graphs,
+                           "parallelism": "single-gpu"},
+            }
+    record["points"] = points
+    print(json.dumps(record))
+    return 0
+
+
 def main() -> int:
     parser = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
     parser.add_argument("--gpus", type=int, default=1)
@@ -309,6 +415,9 @@ def main() -> int:
     parser.add_argument("--no-peaks", action="store_true", help="skip the probes of this device's own peaks")
     parser.add_argument("--mixed", action="store_true",
                         help="also time a step of --batch decoded tokens beside a 2,048-token prompt portion")
+    parser.add_argument("--design", choices=("qwen3", "vupuzen"), default="qwen3",
+                        help="vupuzen: that design beside Qwen3 at equal sizes instead of the default workload")
+    parser.add_argument("--design-shapes", default="", help="with --design vupuzen: further shapes, with commas")
     parser.add_argument("--prefill-only", action="store_true",
                         help="only the prefill measurement (for profiling); prints its part of the record")
     args = parser.parse_args()
@@ -322,6 +431,8 @@ def main() -> int:
         return 1
     from pylon_amd.engine import Runner
 
+    if args.design != "qwen3":
+        return design_main(args)
     shape = dict(SHAPES[args.shape])
     if args.context_length:
         shape["max_position_embeddings"] = args.context_length

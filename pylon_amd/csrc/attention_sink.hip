@@ -16,9 +16,12 @@
 // already laid out as the operand of O^T = V^T P^T.  Scores, bias, maximum, exponentials and
 // sums are float; the weights enter the value product as two bfloat16 terms, p = hi + lo, so
 // that they carry sixteen bits of mantissa.  The sink is where the walk starts: maximum 0,
-// sum 1, output 0.  The waves of a workgroup take heads of one key/value head, so that the keys
-// and values one of them fetched are in the nearest cache for the others.  The order of a
-// query's sums depends on its position only.
+// sum 1, output 0.  The waves of a workgroup take heads of one key/value head at the same
+// tokens: a block's keys and values are fetched once, with 16-byte loads of whole rows, into LDS
+// and read from there by every wave as operands (rows padded against bank conflicts).  Keys
+// may be cut over `cuts` workgroups, which then leave float partial results (maximum, sum,
+// unnormalised output) for a second small kernel to merge in order; the sink belongs to the
+// first cut.  The order of a query's sums depends on its position and the number of cuts only.
 #include "common.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -40,27 +43,35 @@ __global__ __launch_bounds__(256) void attention_sink_kernel(
     bf16_t* __restrict__ out, const bf16_t* __restrict__ q, long long q_stride, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, const int* __restrict__ block_table, int table_width,
     const int* __restrict__ tiles, const int* __restrict__ positions, int n_heads, int n_kv_heads, int dim, int vdim, int page_size, float scale,
-    const float* __restrict__ rel, const int* __restrict__ bucket, int bucket_len, int sink, int waves_per_group) {
-  extern __shared__ float bias_lds[];  // [waves][bucket_len]
+    const float* __restrict__ rel, const int* __restrict__ bucket, int bucket_len, int sink, int waves_per_group,
+    int cuts, float* __restrict__ partial) {
+  extern __shared__ float bias_lds[];  // [waves][bucket_len], then the block's keys and values
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int col = lane & 15, grp = lane >> 4;
   const int group = n_heads / n_kv_heads;
   const int chunks = (group + waves_per_group - 1) / waves_per_group;
   int b = blockIdx.x;
+  const int cut = b % cuts;
+  b /= cuts;
   const int chunk = b % chunks;
   b /= chunks;
   const int kvh = b % n_kv_heads;
   const int tile = b / n_kv_heads;
   const int in_group = chunk * waves_per_group + wave;
-  if (in_group >= group) return;  // no barrier below: a wave may leave alone
-  const int head = kvh * group + in_group;
+  const bool idle = in_group >= group;  // a wave beyond the group's heads helps to fetch and stores nothing
+  const int head = kvh * group + (idle ? group - 1 : in_group);
   // without a table of tiles every token is a tile of its own and row t of the block table is token t's
   const int tok0 = tiles ? tiles[4 * tile] : tile, count = tiles ? tiles[4 * tile + 1] : 1;
   const int row = tiles ? tiles[4 * tile + 2] : tile, pos0 = tiles ? tiles[4 * tile + 3] : positions[tile];
   const int kv_last = pos0 + count - 1;
   const int* table = block_table + static_cast<size_t>(row) * table_width;
 
-  float* tbl = bias_lds + wave * bucket_len;
+  const int tstride = (bucket_len + 3) & ~3;  // keeps what follows the tables 16-byte aligned
+  float* tbl = bias_lds + wave * tstride;
+  const int kstr = dim + 8, vstr = AS_BLOCK + 4;  // LDS rows, padded
+  bf16_t* k_lds = reinterpret_cast<bf16_t*>(bias_lds + waves_per_group * tstride);
+  bf16_t* v_lds = k_lds + AS_BLOCK * kstr;
+  const int threads = waves_per_group * 64;
   if (rel != nullptr)
     for (int d = lane; d < bucket_len; d += 64) tbl[d] = rel[static_cast<size_t>(bucket[d]) * n_heads + head];
   const float far_bias = rel != nullptr ? rel[static_cast<size_t>(bucket[bucket_len - 1]) * n_heads + head] : 0.f;
@@ -88,21 +99,42 @@ __global__ __launch_bounds__(256) void attention_sink_kernel(
 #pragma unroll
   for (int qt = 0; qt < AS_QT; ++qt) {
     // the sink: a key of score 0 without a value (one lane of a query's four carries its one)
-    m_run[qt] = sink ? 0.f : -INFINITY;
-    l_run[qt] = (sink && grp == 0) ? 1.f : 0.f;
+    m_run[qt] = (sink && cut == 0) ? 0.f : -INFINITY;
+    l_run[qt] = (sink && cut == 0 && grp == 0) ? 1.f : 0.f;
 #pragma unroll
     for (int dt = 0; dt < NV; ++dt) o[qt][dt] = floatx4{0.f, 0.f, 0.f, 0.f};
   }
 
-  for (int kb = 0; kb <= kv_last; kb += AS_BLOCK) {
+  const int n_blocks = kv_last / AS_BLOCK + 1;
+  const int per_cut = (n_blocks + cuts - 1) / cuts;
+  const int kb_begin = cut * per_cut * AS_BLOCK;
+  const int kb_end = (cut + 1) * per_cut < n_blocks ? (cut + 1) * per_cut * AS_BLOCK : n_blocks * AS_BLOCK;
+  for (int kb = kb_begin; kb < kb_end; kb += AS_BLOCK) {
     const int page = table[kb / page_size];
     const int in_page = kb % page_size;
+    __syncthreads();  // everybody has read the block before
+    {
+      const int kchunks = dim >> 3;  // 16-byte pieces of a key row
+      const bf16_t* kbase = k_cache + ((static_cast<size_t>(page) * page_size + in_page) * n_kv_heads + kvh) * dim;
+      for (int c = threadIdx.x; c < AS_BLOCK * kchunks; c += threads) {
+        const int r = c / kchunks, e = (c - r * kchunks) * 8;
+        *reinterpret_cast<u32x4*>(k_lds + r * kstr + e) =
+            *reinterpret_cast<const u32x4*>(kbase + static_cast<size_t>(r) * n_kv_heads * dim + e);
+      }
+      const bf16_t* vbase = v_cache + (static_cast<size_t>(page) * n_kv_heads + kvh) * vdim * page_size + in_page;
+      for (int c = threadIdx.x; c < vdim * (AS_BLOCK / 8); c += threads) {
+        const int r = c / (AS_BLOCK / 8), e = (c - r * (AS_BLOCK / 8)) * 8;
+        const u32x4 raw = *reinterpret_cast<const u32x4*>(vbase + static_cast<size_t>(r) * page_size + e);
+        *reinterpret_cast<u32x2*>(v_lds + r * vstr + e) = u32x2{raw[0], raw[1]};
+        *reinterpret_cast<u32x2*>(v_lds + r * vstr + e + 4) = u32x2{raw[2], raw[3]};
+      }
+    }
+    __syncthreads();
     // K operands: row = key, eight elements per lane and step
     floatx4 s[AS_QT][2];
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
-      const size_t slot = static_cast<size_t>(page) * page_size + in_page + t * 16 + col;
-      const bf16_t* kr = k_cache + (slot * n_kv_heads + kvh) * dim;
+      const bf16_t* kr = k_lds + (t * 16 + col) * kstr;
 #pragma unroll
       for (int qt = 0; qt < AS_QT; ++qt) s[qt][t] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -124,8 +156,7 @@ __global__ __launch_bounds__(256) void attention_sink_kernel(
       const int d = dt * 16 + col;
       u32x4 raw = {0u, 0u, 0u, 0u};
       if (d < vdim) {
-        const bf16_t* vr = v_cache + ((static_cast<size_t>(page) * n_kv_heads + kvh) * vdim + d) * page_size +
-                           in_page + 4 * grp;
+        const bf16_t* vr = v_lds + d * vstr + 4 * grp;
         const u32x2 first = *reinterpret_cast<const u32x2*>(vr);
         const u32x2 second = *reinterpret_cast<const u32x2*>(vr + 16);
         raw = u32x4{first[0], first[1], second[0], second[1]};
@@ -198,7 +229,21 @@ __global__ __launch_bounds__(256) void attention_sink_kernel(
     l += __shfl_xor(l, 16, 64);
     l += __shfl_xor(l, 32, 64);
     const int qi = qt * 16 + col;
-    if (qi >= count) continue;
+    if (qi >= count || idle) continue;
+    if (cuts > 1) {
+      // [token, head, cut, 2 + vdim]: maximum, sum, unnormalised output
+      float* dst = partial + ((static_cast<size_t>(tok0 + qi) * n_heads + head) * cuts + cut) * (2 + vdim);
+      if (grp == 0) {
+        dst[0] = m_run[qt];
+        dst[1] = l;
+      }
+#pragma unroll
+      for (int dt = 0; dt < NV; ++dt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (dt * 16 + 4 * grp + i < vdim) dst[2 + dt * 16 + 4 * grp + i] = o[qt][dt][i];
+      continue;
+    }
     const float inv = 1.0f / l;
     bf16_t* orow = out + (static_cast<size_t>(tok0 + qi) * n_heads + head) * vdim;
 #pragma unroll
@@ -216,6 +261,31 @@ __global__ __launch_bounds__(256) void attention_sink_kernel(
   }
 }
 
+// One wave per (token, head): out = sum_c o_c e^(m_c - m) / sum_c l_c e^(m_c - m), cuts in order.
+__global__ void attention_sink_merge_kernel(bf16_t* __restrict__ out, const float* __restrict__ partial, int items,
+                                            int cuts, int vdim) {
+  const int item = blockIdx.x * (blockDim.x / 64) + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (item >= items) return;
+  const float* src = partial + static_cast<size_t>(item) * cuts * (2 + vdim);
+  float m = -INFINITY;
+  for (int c = 0; c < cuts; ++c) m = fmaxf(m, src[c * (2 + vdim)]);
+  float l = 0.f;
+  for (int c = 0; c < cuts; ++c) {
+    const float mc = src[c * (2 + vdim)];
+    if (mc != -INFINITY) l += src[c * (2 + vdim) + 1] * __expf(mc - m);
+  }
+  const float inv = 1.0f / l;
+  for (int d = lane; d < vdim; d += 64) {
+    float acc = 0.f;
+    for (int c = 0; c < cuts; ++c) {
+      const float mc = src[c * (2 + vdim)];
+      if (mc != -INFINITY) acc += src[c * (2 + vdim) + 2 + d] * __expf(mc - m);
+    }
+    out[static_cast<size_t>(item) * vdim + d].bits = float_to_bf16_bits(acc * inv);
+  }
+}
+
 // q: bf16 [tokens, n_heads, dim], rows q_stride elements apart; out: bf16 [tokens, n_heads, vdim].
 // k_cache: bf16 [pages * page_size, n_kv_heads, dim]; v_cache: bf16 [pages, n_kv_heads, vdim, page_size].
 // tiles: int [n_tiles, 4] = (first token, count <= 32, block-table row, first position) of runs of
@@ -227,6 +297,7 @@ extern "C" int pylon_attention_sink(void* out, const void* q, long long q_stride
                                     const void* v_cache, const int* block_table, int table_width, const int* tiles,
                                     const int* positions, int n_tiles, int n_heads, int n_kv_heads, int dim, int vdim, int page_size,
                                     float scale, const float* rel, const int* bucket, int bucket_len, int sink,
+                                    int cuts, float* partial, long long partial_floats, int tokens,
                                     hipStream_t stream) {
   PYLON_REQUIRE(n_tiles >= 0 && n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
                 "attention_sink: %d query heads cannot be grouped over %d key/value heads", n_heads, n_kv_heads);
@@ -241,19 +312,26 @@ extern "C" int pylon_attention_sink(void* out, const void* q, long long q_stride
   PYLON_REQUIRE(tiles != nullptr || positions != nullptr, "attention_sink: tiles or positions are required");
   PYLON_REQUIRE(rel == nullptr || (bucket != nullptr && bucket_len >= 1 && bucket_len <= AS_MAX_BIAS),
                 "attention_sink: a bias by distance needs a table of 1 to %d buckets", AS_MAX_BIAS);
+  PYLON_REQUIRE(cuts >= 1 && cuts <= 64, "attention_sink: 1 to 64 cuts, got %d", cuts);
+  PYLON_REQUIRE(cuts == 1 || (partial != nullptr &&
+                              partial_floats >= static_cast<long long>(tokens) * n_heads * cuts * (2 + vdim)),
+                "attention_sink: cut keys need room for their partial results");
   if (n_tiles == 0) return 0;
   const int group = n_heads / n_kv_heads;
   const int waves = group < 4 ? group : 4;
   const int chunks = (group + waves - 1) / waves;
-  const long long blocks = static_cast<long long>(n_tiles) * n_kv_heads * chunks;
+  const long long blocks = static_cast<long long>(n_tiles) * n_kv_heads * chunks * cuts;
   PYLON_REQUIRE(blocks < (1ll << 31), "attention_sink: too many tiles for one launch");
   dim3 grid(static_cast<unsigned>(blocks)), block(64 * waves);
-  const size_t lds = rel != nullptr ? sizeof(float) * waves * bucket_len : 0;
+  const int table_len = rel != nullptr ? bucket_len : 1;
+  const size_t lds = sizeof(float) * waves * ((table_len + 3) & ~3) + 2 * (static_cast<size_t>(AS_BLOCK) * (dim + 8) +
+                                                              static_cast<size_t>((vdim + 15) / 16 * 16) * (AS_BLOCK + 4));
+  PYLON_REQUIRE(lds <= 160 * 1024, "attention_sink: the bias table and a block do not fit LDS");
   const int ks = (dim + 31) / 32, nv = (vdim + 15) / 16;
 #define GO(KS, NV)                                                                                                 \
   hipLaunchKernelGGL((attention_sink_kernel<KS, NV>), grid, block, lds, stream, (bf16_t*)out, (const bf16_t*)q,     \
                      q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, table_width, tiles,      \
-                     positions, n_heads, n_kv_heads, dim, vdim, page_size, scale, rel, bucket, rel ? bucket_len : 1, sink, waves)
+                     positions, n_heads, n_kv_heads, dim, vdim, page_size, scale, rel, bucket, table_len, sink, waves, cuts, partial)
 #define PICK_NV(KS)                 \
   do {                              \
     if (nv <= 2) GO(KS, 2);         \
@@ -267,5 +345,10 @@ extern "C" int pylon_attention_sink(void* out, const void* q, long long q_stride
   else PICK_NV(8);
 #undef PICK_NV
 #undef GO
+  if (cuts > 1) {
+    const int items = tokens * n_heads;
+    hipLaunchKernelGGL(attention_sink_merge_kernel, dim3((items + 3) / 4), dim3(256), 0, stream, (bf16_t*)out, partial,
+                       items, cuts, vdim);
+  }
   PYLON_LAUNCHED("attention_sink");
 }

@@ -14,8 +14,8 @@
 // so a request's results do not depend on how it was cut into steps or what shared a step.
 #include "common.h"
 
-template <typename T, int NI>
-__global__ void retention_recurrent_kernel(T* __restrict__ out, const T* __restrict__ proj, long long ld,
+template <typename T, int NI, int THREADS>
+__global__ __launch_bounds__(THREADS) void retention_recurrent_kernel(T* __restrict__ out, const T* __restrict__ proj, long long ld,
                                            int q_off, int k_off, int v_off, int g_off, float* state,
                                            const float* __restrict__ decay, const float* __restrict__ inv_freq,
                                            int rot_dims, const int* __restrict__ positions,
@@ -122,7 +122,12 @@ extern "C" int pylon_retention_recurrent(void* out, const void* proj, int dtype,
   dim3 grid(rows, heads), block((vdim * ip_count + PYLON_WAVE - 1) / PYLON_WAVE * PYLON_WAVE);
   const size_t lds = sizeof(float) * (2 * dim + ip_count * vdim + 16);
 #define GO(T, NI)                                                                                              \
-  hipLaunchKernelGGL((retention_recurrent_kernel<T, NI>), grid, block, lds, stream, (T*)out, (const T*)proj, ld, \
+  if (block.x <= 256)                                                                                          \
+    hipLaunchKernelGGL((retention_recurrent_kernel<T, NI, 256>), grid, block, lds, stream, (T*)out, (const T*)proj, ld, \
+                       q_off, k_off, v_off, g_off, state, decay, inv_freq, rot_dims, positions, row_start,      \
+                       row_slots, heads, dim, vdim, ip_count, eps, k_scale);                                    \
+  else                                                                                                         \
+    hipLaunchKernelGGL((retention_recurrent_kernel<T, NI, 1024>), grid, block, lds, stream, (T*)out, (const T*)proj, ld, \
                      q_off, k_off, v_off, g_off, state, decay, inv_freq, rot_dims, positions, row_start,        \
                      row_slots, heads, dim, vdim, ip_count, eps, k_scale)
 #define PICK(T)                 \

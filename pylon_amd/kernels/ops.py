@@ -251,14 +251,29 @@ def attention_sink_ok(dtype: torch.dtype, *, head_dim: int, v_dim: int, page_siz
             and 4 <= v_dim <= 256 and page_size % 32 == 0 and bucket_len <= SINK_MAX_BIAS and window is None)
 
 
+def sink_cuts(tokens: int, n_heads: int, n_kv_heads: int, max_len: int, units: Optional[int] = None) -> int:
+    """Workgroups that share the keys of one (token, key/value head) in a step of single tokens:
+    more than one while the launch would leave compute units idle and every cut keeps at least
+    256 keys of the longest request (``max_len`` may be an upper bound)."""
+    units = units or _lib.compute_units()
+    group = n_heads // n_kv_heads
+    groups = tokens * n_kv_heads * (-(-group // min(4, group)))
+    cuts = 1
+    while cuts < 64 and groups * cuts * 2 <= 2 * units and max_len >= cuts * 2 * 256:
+        cuts *= 2
+    return cuts
+
+
 def attention_sink(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
                    tiles: Optional[torch.Tensor], positions: Optional[torch.Tensor], *, page_size: int, scale: float,
-                   rel: Optional[torch.Tensor], bucket: Optional[torch.Tensor], sink: bool) -> torch.Tensor:
+                   rel: Optional[torch.Tensor], bucket: Optional[torch.Tensor], sink: bool,
+                   cuts: int = 1) -> torch.Tensor:
     """Causal attention with a bias by distance and a sink on the matrix cores: bfloat16 ``q``
     ``[tokens, heads, head_dim]`` (maybe a slice of wider rows), keys ``[pages, page_size, kv_heads,
     head_dim]``, values transposed inside their pages ``[pages, kv_heads, v_dim, page_size]``.
     ``tiles`` int32 ``[n, 4]`` (first token, count <= 32, block-table row, first position); or None
-    with ``positions``: every token a tile of its own on its own row of the table."""
+    with ``positions``: every token a tile of its own on its own row of the table.  ``cuts``
+    workgroups share the keys of a tile and a second kernel merges their float partial results."""
     if q.dim() != 3 or k_cache.dim() != 4 or v_cache.dim() != 4:
         raise KernelError("attention_sink takes q [tokens, heads, head_dim] and 4-D caches")
     tokens, n_heads, head_dim = q.shape
@@ -286,11 +301,15 @@ def attention_sink(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
             raise KernelError("attention_sink: without tiles, one position and one table row per token")
         n_tiles = tokens
     out = torch.empty((tokens, n_heads, v_dim), dtype=q.dtype, device=q.device)
+    partial = None
+    if cuts > 1:
+        partial = torch.empty((tokens * n_heads * cuts * (2 + v_dim),), dtype=torch.float32, device=q.device)
     _lib.call("pylon_attention_sink", _dev(out, "out"), q.data_ptr(), q.stride(0) if tokens > 1 else n_heads * head_dim,
               _dev(k_cache, "k_cache"), _dev(v_cache, "v_cache"), _dev(block_table, "block_table", torch.int32),
               block_table.shape[1], _dev(tiles, "tiles", torch.int32), _dev(positions, "positions", torch.int32),
               n_tiles, n_heads, n_kv_heads, head_dim, v_dim, page_size, float(scale), _dev(rel, "rel", torch.float32),
-              _dev(bucket, "bucket", torch.int32), 0 if bucket is None else bucket.numel(), 1 if sink else 0, _stream())
+              _dev(bucket, "bucket", torch.int32), 0 if bucket is None else bucket.numel(), 1 if sink else 0,
+              int(cuts), _dev(partial, "partial"), 0 if partial is None else partial.numel(), tokens, _stream())
     return out
 
 

@@ -177,8 +177,17 @@ class SinkAttention(Part):
         spec = self.spec
         return KVRequirement(spec.n_kv_heads, spec.head_dim, spec.window, v_head_dim=spec.v_head_dim)
 
+    def _matrix_cores(self, page_size: int) -> bool:
+        spec = self.spec
+        return ops.attention_sink_ok(self.dtype, head_dim=spec.head_dim, v_dim=spec.v_head_dim, page_size=page_size,
+                                     bucket_len=self.bucket.numel(), window=spec.window)
+
     def decode_signature(self, rows: int, bound: int) -> tuple:
-        return ("sink_attention",)  # one wave per (token, head), whatever the lengths
+        """Of a bound on the lengths a step of single tokens takes only over how many workgroups
+        a request's keys are cut."""
+        if self.dtype != torch.bfloat16:
+            return ("sink_attention",)
+        return ("sink_attention", ops.sink_cuts(rows, self.spec.n_heads, self.spec.n_kv_heads, bound))
 
     def forward(self, h: torch.Tensor, ctx, cache, stores: bool) -> torch.Tensor:
         spec = self.spec
@@ -191,12 +200,12 @@ class SinkAttention(Part):
             ops.kv_store(qkv, cache.k, v_cache, cache.slot_map, k_off=self.q_size, v_off=self.q_size + self.k_size,
                          v_transposed=True)
         q = qkv.as_strided((tokens, spec.n_heads, spec.head_dim), (qkv.stride(0), spec.head_dim, 1))
-        if ops.attention_sink_ok(self.dtype, head_dim=spec.head_dim, v_dim=spec.v_head_dim, page_size=page_size,
-                                 bucket_len=self.bucket.numel(), window=spec.window) and qkv.stride(0) % 8 == 0:
+        if self._matrix_cores(page_size) and qkv.stride(0) % 8 == 0:
             tiles = None if ctx.decode_only else ctx.token_tiles(ops.SINK_TILE)
+            cuts = ops.sink_cuts(tokens, spec.n_heads, spec.n_kv_heads, ctx.max_len) if ctx.decode_only else 1
             context = ops.attention_sink(q, cache.k, v_cache, cache.block_table, tiles, ctx.positions,
                                          page_size=page_size, scale=spec.scale, rel=self.params["rel"],
-                                         bucket=self.bucket, sink=spec.sink)
+                                         bucket=self.bucket, sink=spec.sink, cuts=cuts)
         else:
             context = ops.paged_attention(
                 q, cache.k, v_cache, cache.block_table, ctx.tok_row, ctx.positions, page_size=page_size,

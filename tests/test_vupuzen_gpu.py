@@ -247,9 +247,13 @@ def test_sink_attention_on_the_matrix_cores(ops, dim, vdim, heads, groups, rows,
     lengths = [total, 33, 1]
     table[0], table[2] = table[1], table[1]
     singles = torch.tensor(np.stack([q[n - 1] for n in lengths]), dtype=torch.bfloat16, device=DEV)
-    got = ops.attention_sink(singles, kc, vt, table, None, i32([n - 1 for n in lengths]), **common).float().cpu().numpy()
-    for r, n in enumerate(lengths):
-        assert np.abs(got[r] - want[n - 1]).max() < 2e-2 * max(1.0, np.abs(want).max()), n
+    for cuts in (1, 2, 8):  # the keys of a request shared between workgroups, merged by a second kernel
+        got = ops.attention_sink(singles, kc, vt, table, None, i32([n - 1 for n in lengths]), cuts=cuts,
+                                 **common).float().cpu().numpy()
+        for r, n in enumerate(lengths):
+            assert np.abs(got[r] - want[n - 1]).max() < 2e-2 * max(1.0, np.abs(want).max()), (n, cuts)
+    assert ops.sink_cuts(8, 32, 8, 128, units=256) == 1 and ops.sink_cuts(8, 32, 8, 2048, units=256) == 8
+    assert ops.sink_cuts(1, 32, 8, 100000, units=256) == 64 and ops.sink_cuts(64, 32, 8, 100000, units=256) == 1
 
 
 def test_a_sink_takes_all_the_weight_when_every_score_is_far_below_zero(ops):
