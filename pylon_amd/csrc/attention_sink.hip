@@ -1,10 +1,10 @@
 // Paged causal attention with a learned bias by distance and a sink, on the matrix cores, for
 // bfloat16 prompt portions and single tokens alike:
 //
-//   s_ij = scale * q_i.k_j + rel[bucket[min(i - j, bucket_len - 1)], head],   j <= i
+//   s_ij = scale * q_i.k_j + bias[head, min(i - j, bucket_len - 1)],   j <= i
 //   out_i = sum_j exp(s_ij) v_j / (1 + sum_j exp(s_ij))
 //
-// Keys have `dim` elements, values `vdim`.  Keys lie in the cache as [slot, kv head, dim];
+// (the learned table's rows already looked up by distance).  Keys have `dim` elements, values `vdim`.  Keys lie in the cache as [slot, kv head, dim];
 // values lie transposed inside every page, [page, kv head, vdim, slot in page], so that the
 // eight keys a lane feeds to a matrix instruction are neighbours in memory.
 //
@@ -43,8 +43,9 @@ __global__ __launch_bounds__(256) void attention_sink_kernel(
     bf16_t* __restrict__ out, const bf16_t* __restrict__ q, long long q_stride, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, const int* __restrict__ block_table, int table_width,
     const int* __restrict__ tiles, const int* __restrict__ positions, int n_heads, int n_kv_heads, int dim, int vdim, int page_size, float scale,
-    const float* __restrict__ rel, const int* __restrict__ bucket, int bucket_len, int sink, int waves_per_group,
-    int cuts, float* __restrict__ partial) {
+    const float* __restrict__ bias, int bucket_len, int sink, int cuts, float* __restrict__ partial) {
+  constexpr int waves_per_group = 4;
+  constexpr int KL = (KS + 1) / 2, VL = (NV + 3) / 4;  // 16-byte pieces of a block a thread fetches
   extern __shared__ float bias_lds[];  // [waves][bucket_len], then the block's keys and values
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int col = lane & 15, grp = lane >> 4;
@@ -64,6 +65,7 @@ __global__ __launch_bounds__(256) void attention_sink_kernel(
   const int tok0 = tiles ? tiles[4 * tile] : tile, count = tiles ? tiles[4 * tile + 1] : 1;
   const int row = tiles ? tiles[4 * tile + 2] : tile, pos0 = tiles ? tiles[4 * tile + 3] : positions[tile];
   const int kv_last = pos0 + count - 1;
+  const int n_qt = count > 16 ? AS_QT : 1;  // a tile of up to 16 tokens (a single token, a portion's end) needs one
   const int* table = block_table + static_cast<size_t>(row) * table_width;
 
   const int tstride = (bucket_len + 3) & ~3;  // keeps what follows the tables 16-byte aligned
@@ -71,10 +73,13 @@ __global__ __launch_bounds__(256) void attention_sink_kernel(
   const int kstr = dim + 8, vstr = AS_BLOCK + 4;  // LDS rows, padded
   bf16_t* k_lds = reinterpret_cast<bf16_t*>(bias_lds + waves_per_group * tstride);
   bf16_t* v_lds = k_lds + AS_BLOCK * kstr;
-  const int threads = waves_per_group * 64;
-  if (rel != nullptr)
-    for (int d = lane; d < bucket_len; d += 64) tbl[d] = rel[static_cast<size_t>(bucket[d]) * n_heads + head];
-  const float far_bias = rel != nullptr ? rel[static_cast<size_t>(bucket[bucket_len - 1]) * n_heads + head] : 0.f;
+  constexpr int threads = waves_per_group * 64;
+  const float* bias_row = bias ? bias + static_cast<size_t>(head) * bucket_len : nullptr;
+  if (bias != nullptr) {
+#pragma unroll 8
+    for (int d = lane; d < bucket_len; d += 64) tbl[d] = bias_row[d];
+  }
+  const float far_bias = bias != nullptr ? bias_row[bucket_len - 1] : 0.f;
 
   // Q^T operands: column = query, eight key elements per lane and step
   bf16x8 qf[AS_QT][KS];
@@ -109,27 +114,57 @@ __global__ __launch_bounds__(256) void attention_sink_kernel(
   const int per_cut = (n_blocks + cuts - 1) / cuts;
   const int kb_begin = cut * per_cut * AS_BLOCK;
   const int kb_end = (cut + 1) * per_cut < n_blocks ? (cut + 1) * per_cut * AS_BLOCK : n_blocks * AS_BLOCK;
-  for (int kb = kb_begin; kb < kb_end; kb += AS_BLOCK) {
+  // A block's keys and values travel global -> registers -> LDS; the registers of block b + 1
+  // are filled while block b is computed.
+  u32x4 kreg[KL], vreg[VL];
+  const int kchunks = dim >> 3;  // 16-byte pieces of a key row
+  auto fetch = [&](int kb) {
     const int page = table[kb / page_size];
     const int in_page = kb % page_size;
-    __syncthreads();  // everybody has read the block before
-    {
-      const int kchunks = dim >> 3;  // 16-byte pieces of a key row
-      const bf16_t* kbase = k_cache + ((static_cast<size_t>(page) * page_size + in_page) * n_kv_heads + kvh) * dim;
-      for (int c = threadIdx.x; c < AS_BLOCK * kchunks; c += threads) {
+    const bf16_t* kbase = k_cache + ((static_cast<size_t>(page) * page_size + in_page) * n_kv_heads + kvh) * dim;
+#pragma unroll
+    for (int n = 0; n < KL; ++n) {
+      const int c = threadIdx.x + n * threads;
+      if (c < AS_BLOCK * kchunks) {
         const int r = c / kchunks, e = (c - r * kchunks) * 8;
-        *reinterpret_cast<u32x4*>(k_lds + r * kstr + e) =
-            *reinterpret_cast<const u32x4*>(kbase + static_cast<size_t>(r) * n_kv_heads * dim + e);
-      }
-      const bf16_t* vbase = v_cache + (static_cast<size_t>(page) * n_kv_heads + kvh) * vdim * page_size + in_page;
-      for (int c = threadIdx.x; c < vdim * (AS_BLOCK / 8); c += threads) {
-        const int r = c / (AS_BLOCK / 8), e = (c - r * (AS_BLOCK / 8)) * 8;
-        const u32x4 raw = *reinterpret_cast<const u32x4*>(vbase + static_cast<size_t>(r) * page_size + e);
-        *reinterpret_cast<u32x2*>(v_lds + r * vstr + e) = u32x2{raw[0], raw[1]};
-        *reinterpret_cast<u32x2*>(v_lds + r * vstr + e + 4) = u32x2{raw[2], raw[3]};
+        kreg[n] = *reinterpret_cast<const u32x4*>(kbase + static_cast<size_t>(r) * n_kv_heads * dim + e);
       }
     }
+    const bf16_t* vbase = v_cache + (static_cast<size_t>(page) * n_kv_heads + kvh) * vdim * page_size + in_page;
+#pragma unroll
+    for (int n = 0; n < VL; ++n) {
+      const int c = threadIdx.x + n * threads;
+      if (c < vdim * (AS_BLOCK / 8)) {
+        const int r = c / (AS_BLOCK / 8), e = (c - r * (AS_BLOCK / 8)) * 8;
+        vreg[n] = *reinterpret_cast<const u32x4*>(vbase + static_cast<size_t>(r) * page_size + e);
+      }
+    }
+  };
+  auto stage = [&]() {
+#pragma unroll
+    for (int n = 0; n < KL; ++n) {
+      const int c = threadIdx.x + n * threads;
+      if (c < AS_BLOCK * kchunks) {
+        const int r = c / kchunks, e = (c - r * kchunks) * 8;
+        *reinterpret_cast<u32x4*>(k_lds + r * kstr + e) = kreg[n];
+      }
+    }
+#pragma unroll
+    for (int n = 0; n < VL; ++n) {
+      const int c = threadIdx.x + n * threads;
+      if (c < vdim * (AS_BLOCK / 8)) {
+        const int r = c / (AS_BLOCK / 8), e = (c - r * (AS_BLOCK / 8)) * 8;
+        *reinterpret_cast<u32x2*>(v_lds + r * vstr + e) = u32x2{vreg[n][0], vreg[n][1]};
+        *reinterpret_cast<u32x2*>(v_lds + r * vstr + e + 4) = u32x2{vreg[n][2], vreg[n][3]};
+      }
+    }
+  };
+  if (kb_begin < kb_end) fetch(kb_begin);
+  for (int kb = kb_begin; kb < kb_end; kb += AS_BLOCK) {
+    __syncthreads();  // everybody has read the block before
+    stage();
     __syncthreads();
+    if (kb + AS_BLOCK < kb_end) fetch(kb + AS_BLOCK);
     // K operands: row = key, eight elements per lane and step
     floatx4 s[AS_QT][2];
 #pragma unroll
@@ -145,7 +180,7 @@ __global__ __launch_bounds__(256) void attention_sink_kernel(
         const bf16x8 kf = __builtin_bit_cast(bf16x8, raw);
 #pragma unroll
         for (int qt = 0; qt < AS_QT; ++qt)
-          s[qt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[qt][ks], s[qt][t], 0, 0, 0);
+          if (qt < n_qt) s[qt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[qt][ks], s[qt][t], 0, 0, 0);
       }
     }
     // V^T operands: row = value element, keys kb + 4 grp + {0..3} and kb + 16 + 4 grp + {0..3}
@@ -173,10 +208,11 @@ __global__ __launch_bounds__(256) void attention_sink_kernel(
 
 #pragma unroll
     for (int qt = 0; qt < AS_QT; ++qt) {
+      if (qt >= n_qt) continue;
       // scores of this lane: keys kb + 16 t + 4 grp + i for query qpos[qt]
       float sc[8];
       const int near = qpos[qt] - (kb + AS_BLOCK - 1);  // the smallest distance of the block for this query
-      const bool all_far = rel == nullptr || near >= bucket_len - 1;
+      const bool all_far = bias == nullptr || near >= bucket_len - 1;
       float top = m_run[qt];
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
@@ -208,15 +244,20 @@ __global__ __launch_bounds__(256) void attention_sink_kernel(
       u32x4 hi, lo;
 #pragma unroll
       for (int e = 0; e < 8; e += 2) {
-        const uint32_t h = as_pack(p[e], p[e + 1]);
-        hi[e >> 1] = h;
-        lo[e >> 1] = as_pack(p[e] - __uint_as_float(h << 16), p[e + 1] - __uint_as_float(h & 0xffff0000u));
+        // hi: the upper sixteen bits of p as they are; lo: those of the rest (p - hi is exact)
+        const uint32_t a = __float_as_uint(p[e]), c = __float_as_uint(p[e + 1]);
+        hi[e >> 1] = __builtin_amdgcn_perm(c, a, 0x07060302u);
+        const float ra = p[e] - __uint_as_float(a & 0xffff0000u), rc = p[e + 1] - __uint_as_float(c & 0xffff0000u);
+        lo[e >> 1] = __builtin_amdgcn_perm(__float_as_uint(rc), __float_as_uint(ra), 0x07060302u);
       }
       const bf16x8 p_hi = __builtin_bit_cast(bf16x8, hi), p_lo = __builtin_bit_cast(bf16x8, lo);
+      const bool rescale = __any(corr != 1.f);  // no query of the wave raised its maximum: nothing to scale
 #pragma unroll
       for (int dt = 0; dt < NV; ++dt) {
         floatx4 acc = o[qt][dt];
-        acc[0] *= corr; acc[1] *= corr; acc[2] *= corr; acc[3] *= corr;
+        if (rescale) {
+          acc[0] *= corr; acc[1] *= corr; acc[2] *= corr; acc[3] *= corr;
+        }
         acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], p_hi, acc, 0, 0, 0);
         o[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], p_lo, acc, 0, 0, 0);
       }
@@ -290,13 +331,13 @@ __global__ void attention_sink_merge_kernel(bf16_t* __restrict__ out, const floa
 // k_cache: bf16 [pages * page_size, n_kv_heads, dim]; v_cache: bf16 [pages, n_kv_heads, vdim, page_size].
 // tiles: int [n_tiles, 4] = (first token, count <= 32, block-table row, first position) of runs of
 // consecutive tokens of one request; or null, and then positions: int [n_tiles], one token per tile,
-// token t on row t of the block table (a step of single tokens).  rel: null or float [rows, n_heads] with bucket: int
-// [bucket_len <= 4096] rows of rel by distance.  dim a multiple of 8 up to 256, vdim a multiple of 4
+// token t on row t of the block table (a step of single tokens).  bias: null or float [n_heads, bucket_len
+// <= 4096], a head's bias by distance, the last entry for every distance from bucket_len - 1 on.  dim a multiple of 8 up to 256, vdim a multiple of 4
 // up to 256, page_size a multiple of 32.  The host guarantees that the tiles lie inside q and the table.
 extern "C" int pylon_attention_sink(void* out, const void* q, long long q_stride, const void* k_cache,
                                     const void* v_cache, const int* block_table, int table_width, const int* tiles,
                                     const int* positions, int n_tiles, int n_heads, int n_kv_heads, int dim, int vdim, int page_size,
-                                    float scale, const float* rel, const int* bucket, int bucket_len, int sink,
+                                    float scale, const float* bias, int bucket_len, int sink,
                                     int cuts, float* partial, long long partial_floats, int tokens,
                                     hipStream_t stream) {
   PYLON_REQUIRE(n_tiles >= 0 && n_heads > 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0,
@@ -310,28 +351,33 @@ extern "C" int pylon_attention_sink(void* out, const void* q, long long q_stride
                 (reinterpret_cast<uintptr_t>(v_cache) & 7) == 0 && (reinterpret_cast<uintptr_t>(out) & 7) == 0,
                 "attention_sink: operands must be 16-byte aligned");
   PYLON_REQUIRE(tiles != nullptr || positions != nullptr, "attention_sink: tiles or positions are required");
-  PYLON_REQUIRE(rel == nullptr || (bucket != nullptr && bucket_len >= 1 && bucket_len <= AS_MAX_BIAS),
-                "attention_sink: a bias by distance needs a table of 1 to %d buckets", AS_MAX_BIAS);
+  PYLON_REQUIRE(bias == nullptr || (bucket_len >= 1 && bucket_len <= AS_MAX_BIAS),
+                "attention_sink: a bias by distance is a table of 1 to %d entries a head", AS_MAX_BIAS);
   PYLON_REQUIRE(cuts >= 1 && cuts <= 64, "attention_sink: 1 to 64 cuts, got %d", cuts);
   PYLON_REQUIRE(cuts == 1 || (partial != nullptr &&
                               partial_floats >= static_cast<long long>(tokens) * n_heads * cuts * (2 + vdim)),
                 "attention_sink: cut keys need room for their partial results");
   if (n_tiles == 0) return 0;
   const int group = n_heads / n_kv_heads;
-  const int waves = group < 4 ? group : 4;
+  const int waves = 4;
   const int chunks = (group + waves - 1) / waves;
   const long long blocks = static_cast<long long>(n_tiles) * n_kv_heads * chunks * cuts;
   PYLON_REQUIRE(blocks < (1ll << 31), "attention_sink: too many tiles for one launch");
   dim3 grid(static_cast<unsigned>(blocks)), block(64 * waves);
-  const int table_len = rel != nullptr ? bucket_len : 1;
+  const int table_len = bias != nullptr ? bucket_len : 1;
   const size_t lds = sizeof(float) * waves * ((table_len + 3) & ~3) + 2 * (static_cast<size_t>(AS_BLOCK) * (dim + 8) +
                                                               static_cast<size_t>((vdim + 15) / 16 * 16) * (AS_BLOCK + 4));
   PYLON_REQUIRE(lds <= 160 * 1024, "attention_sink: the bias table and a block do not fit LDS");
   const int ks = (dim + 31) / 32, nv = (vdim + 15) / 16;
-#define GO(KS, NV)                                                                                                 \
-  hipLaunchKernelGGL((attention_sink_kernel<KS, NV>), grid, block, lds, stream, (bf16_t*)out, (const bf16_t*)q,     \
-                     q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, table_width, tiles,      \
-                     positions, n_heads, n_kv_heads, dim, vdim, page_size, scale, rel, bucket, table_len, sink, waves, cuts, partial)
+#define GO(KS, NV) \
+  do { \
+  if (lds > 48 * 1024) \
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_sink_kernel<KS, NV>), \
+                              hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)); \
+  hipLaunchKernelGGL((attention_sink_kernel<KS, NV>), grid, block, lds, stream, (bf16_t*)out, (const bf16_t*)q, \
+                     q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, table_width, tiles, \
+                     positions, n_heads, n_kv_heads, dim, vdim, page_size, scale, bias, table_len, sink, cuts, partial); \
+  } while (0)
 #define PICK_NV(KS)                 \
   do {                              \
     if (nv <= 2) GO(KS, 2);         \

@@ -1,0 +1,326 @@
+// Retention of bfloat16 prompt portions on the matrix cores, in chunks of 32 tokens.  For the
+// tokens 0..n-1 of a chunk, with S the state before it and L the head's decay:
+//
+//   o_i = L^(i+1) S^T q_i + sum_{j <= i} L^(i-j) (q_i . k_j) v_j
+//   S'  = L^n S + sum_j L^(n-1-j) k_j v_j^T
+//
+// (q and k rotated by their positions, k scaled), then out_i = o_i / rms(o_i) * silu(g_i) as in
+// the recurrent form.  One workgroup of four waves per (row of the step, head) walks the row's
+// chunks in order.  The state stays in float accumulators for the whole walk, every wave
+// owning the columns (value elements) of its tiles; everything else of a chunk is staged in LDS.
+// All products run as 16x16x32 bfloat16 instructions with float accumulation, and every float
+// operand (the rotated q and k, the state, the decayed scores, the decayed keys) enters them as
+// two bfloat16 terms, x = hi + lo, products of two such operands as hi*hi + hi*lo + lo*hi: what
+// the design keeps in 32 bits is carried with sixteen bits of mantissa or more; v is the
+// projection's bfloat16 as it is.  Outputs are computed transposed (rows: value elements,
+// columns: tokens), so that a token's norm is a sum within its column's lanes.
+#include "common.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+
+#define RC_CHUNK 32
+#define RC_TSTR (RC_CHUNK + 8)  // row of a [element][token] array in LDS, 16-byte aligned
+
+// Upper halves of two floats side by side (a bfloat16 pair, truncated), and of what is left.
+__device__ __forceinline__ void rc_split(float a, float b, uint32_t& hi, uint32_t& lo) {
+  const uint32_t ua = __float_as_uint(a), ub = __float_as_uint(b);
+  hi = __builtin_amdgcn_perm(ub, ua, 0x07060302u);
+  const float ra = a - __uint_as_float(ua & 0xffff0000u), rb = b - __uint_as_float(ub & 0xffff0000u);
+  lo = __builtin_amdgcn_perm(__float_as_uint(rb), __float_as_uint(ra), 0x07060302u);
+}
+__device__ __forceinline__ void rc_split1(float a, uint16_t& hi, uint16_t& lo) {
+  const uint32_t ua = __float_as_uint(a);
+  hi = static_cast<uint16_t>(ua >> 16);
+  lo = static_cast<uint16_t>(__float_as_uint(a - __uint_as_float(ua & 0xffff0000u)) >> 16);
+}
+
+#define RC_MFMA(a, b, c) __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0)
+
+// KS: slabs of 32 key elements (dim = 32 KS); NVW: tiles of 16 value elements per wave (vdim <= 64 NVW).
+template <int KS, int NVW>
+__global__ __launch_bounds__(256) void retention_chunked_kernel(
+    bf16_t* __restrict__ out, const bf16_t* __restrict__ proj, long long ld, int q_off, int k_off, int v_off, int g_off,
+    float* state, const float* __restrict__ decay, const float* __restrict__ inv_freq, int rot_dims,
+    const int* __restrict__ positions, const int* __restrict__ row_start, const int* __restrict__ row_slots,
+    int heads, int vdim, float eps, float k_scale) {
+  constexpr int dim = 32 * KS, ND = 2 * KS;
+  constexpr int QSTR = dim + 8;  // row of a [token][element] array in LDS
+  extern __shared__ uint16_t rc_lds[];
+  uint16_t* q_hi = rc_lds;                      // [32][QSTR]
+  uint16_t* q_lo = q_hi + RC_CHUNK * QSTR;
+  uint16_t* k_hi = q_lo + RC_CHUNK * QSTR;
+  uint16_t* k_lo = k_hi + RC_CHUNK * QSTR;
+  uint16_t* kw_hi = k_lo + RC_CHUNK * QSTR;     // [dim][RC_TSTR]: decayed keys, transposed
+  uint16_t* kw_lo = kw_hi + dim * RC_TSTR;
+  uint16_t* v_t = kw_lo + dim * RC_TSTR;        // [vdim16][RC_TSTR]: values, transposed
+  const int vdim16 = (vdim + 15) & ~15;
+  float* red = reinterpret_cast<float*>(v_t + vdim16 * RC_TSTR);  // [4][32]
+
+  const int row = blockIdx.x, head = blockIdx.y;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int col = lane & 15, grp = lane >> 4;
+  const int begin = row_start[row], end = row_start[row + 1];
+  float* st = state + ((static_cast<size_t>(row_slots[row]) * heads + head) * dim) * vdim;
+  const float lam = decay[head];
+  const float log2lam = log2f(lam);
+  const int half = rot_dims / 2;
+  const int n_vt = vdim16 / 16;
+
+  // S[d tile][own value tile]: column = value element, rows = key elements 4 grp + i
+  floatx4 s[ND][NVW];
+#pragma unroll
+  for (int n = 0; n < NVW; ++n) {
+    const int e = (wave + 4 * n) * 16 + col;
+#pragma unroll
+    for (int dt = 0; dt < ND; ++dt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        s[dt][n][i] = (e < vdim) ? st[static_cast<size_t>(dt * 16 + 4 * grp + i) * vdim + e] : 0.f;
+  }
+
+  for (int c0 = begin; c0 < end; c0 += RC_CHUNK) {
+    const int n_tok = end - c0 < RC_CHUNK ? end - c0 : RC_CHUNK;
+    // ---- stage the chunk: rotated q and k as two terms, decayed keys transposed, values transposed
+    for (int idx = tid; idx < RC_CHUNK * (dim / 2); idx += 256) {
+      const int tok = idx / (dim / 2), pr = idx - tok * (dim / 2);
+      int d0, d1;
+      if (pr < half) { d0 = pr; d1 = pr + half; } else { d0 = rot_dims + 2 * (pr - half); d1 = d0 + 1; }
+      float q0 = 0.f, q1 = 0.f, k0 = 0.f, k1 = 0.f;
+      if (tok < n_tok) {
+        const bf16_t* pr_row = proj + static_cast<size_t>(c0 + tok) * ld;
+        const bf16_t* qr = pr_row + q_off + head * dim;
+        const bf16_t* kr = pr_row + k_off + head * dim;
+        q0 = to_float(qr[d0]); q1 = to_float(qr[d1]);
+        k0 = to_float(kr[d0]); k1 = to_float(kr[d1]);
+        if (pr < half) {
+          const float angle = static_cast<float>(positions[c0 + tok]) * inv_freq[pr];
+          float sn, cs;
+          sincosf(angle, &sn, &cs);
+          const float a = q0 * cs - q1 * sn, b = q1 * cs + q0 * sn;
+          q0 = a; q1 = b;
+          const float e = k0 * cs - k1 * sn, f = k1 * cs + k0 * sn;
+          k0 = e; k1 = f;
+        }
+        k0 *= k_scale; k1 *= k_scale;
+      }
+      rc_split1(q0, q_hi[tok * QSTR + d0], q_lo[tok * QSTR + d0]);
+      rc_split1(q1, q_hi[tok * QSTR + d1], q_lo[tok * QSTR + d1]);
+      rc_split1(k0, k_hi[tok * QSTR + d0], k_lo[tok * QSTR + d0]);
+      rc_split1(k1, k_hi[tok * QSTR + d1], k_lo[tok * QSTR + d1]);
+      // the key's weight in the state after the chunk: L^(n - 1 - j)
+      const float w = tok < n_tok ? exp2f(static_cast<float>(n_tok - 1 - tok) * log2lam) : 0.f;
+      rc_split1(k0 * w, kw_hi[d0 * RC_TSTR + tok], kw_lo[d0 * RC_TSTR + tok]);
+      rc_split1(k1 * w, kw_hi[d1 * RC_TSTR + tok], kw_lo[d1 * RC_TSTR + tok]);
+    }
+    for (int idx = tid; idx < RC_CHUNK * vdim16; idx += 256) {
+      const int tok = idx / vdim16, e = idx - tok * vdim16;
+      uint16_t bits = 0;
+      if (tok < n_tok && e < vdim) bits = proj[static_cast<size_t>(c0 + tok) * ld + v_off + head * vdim + e].bits;
+      v_t[e * RC_TSTR + tok] = bits;
+    }
+    __syncthreads();
+
+    // ---- decayed scores, transposed: rows = tokens j, columns = tokens i; p[ti] holds for token
+    // i = 16 ti + col the tokens j = 4 grp + i' (first four) and 16 + 4 grp + i' (last four)
+    u32x4 p_hi[2], p_lo[2];
+#pragma unroll
+    for (int ti = 0; ti < 2; ++ti) {
+      float pv[8];
+#pragma unroll
+      for (int tj = 0; tj < 2; ++tj) {
+        floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+        if (tj <= ti) {
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks) {
+            const int off = ks * 32 + grp * 8;
+            const u32x4 kh = *reinterpret_cast<const u32x4*>(k_hi + (tj * 16 + col) * QSTR + off);
+            const u32x4 kl = *reinterpret_cast<const u32x4*>(k_lo + (tj * 16 + col) * QSTR + off);
+            const u32x4 qh = *reinterpret_cast<const u32x4*>(q_hi + (ti * 16 + col) * QSTR + off);
+            const u32x4 ql = *reinterpret_cast<const u32x4*>(q_lo + (ti * 16 + col) * QSTR + off);
+            acc = RC_MFMA(kh, qh, acc);
+            acc = RC_MFMA(kh, ql, acc);
+            acc = RC_MFMA(kl, qh, acc);
+          }
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int dist = (ti * 16 + col) - (tj * 16 + 4 * grp + i);
+          pv[tj * 4 + i] = dist >= 0 ? acc[i] * exp2f(static_cast<float>(dist) * log2lam) : 0.f;
+        }
+      }
+#pragma unroll
+      for (int e = 0; e < 8; e += 2) {
+        uint32_t h, l;
+        rc_split(pv[e], pv[e + 1], h, l);
+        p_hi[ti][e >> 1] = h;
+        p_lo[ti][e >> 1] = l;
+      }
+    }
+
+    // ---- outputs, transposed: rows = value elements of the wave's tiles, columns = tokens
+    floatx4 o[NVW][2];
+#pragma unroll
+    for (int n = 0; n < NVW; ++n) {
+      const int dt_e = wave + 4 * n;
+      o[n][0] = floatx4{0.f, 0.f, 0.f, 0.f};
+      o[n][1] = floatx4{0.f, 0.f, 0.f, 0.f};
+      if (dt_e >= n_vt) continue;
+      // what the state before the chunk gives: S^T q, the key elements of a slab in the order the
+      // accumulators hold them (4 grp + i, then 16 + 4 grp + i)
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        u32x4 sh, sl;
+#pragma unroll
+        for (int e = 0; e < 8; e += 2) {
+          uint32_t h, l;
+          rc_split(s[2 * ks + (e >> 2)][n][e & 3], s[2 * ks + (e >> 2)][n][(e & 3) + 1], h, l);
+          sh[e >> 1] = h;
+          sl[e >> 1] = l;
+        }
+#pragma unroll
+        for (int ti = 0; ti < 2; ++ti) {
+          const uint16_t* qh_row = q_hi + (ti * 16 + col) * QSTR + ks * 32 + 4 * grp;
+          const uint16_t* ql_row = q_lo + (ti * 16 + col) * QSTR + ks * 32 + 4 * grp;
+          const u32x2 a0 = *reinterpret_cast<const u32x2*>(qh_row), a1 = *reinterpret_cast<const u32x2*>(qh_row + 16);
+          const u32x2 b0 = *reinterpret_cast<const u32x2*>(ql_row), b1 = *reinterpret_cast<const u32x2*>(ql_row + 16);
+          const u32x4 qh = {a0[0], a0[1], a1[0], a1[1]}, ql = {b0[0], b0[1], b1[0], b1[1]};
+          o[n][ti] = RC_MFMA(sh, qh, o[n][ti]);
+          o[n][ti] = RC_MFMA(sh, ql, o[n][ti]);
+          o[n][ti] = RC_MFMA(sl, qh, o[n][ti]);
+        }
+      }
+#pragma unroll
+      for (int ti = 0; ti < 2; ++ti) {
+        const float w = exp2f(static_cast<float>(ti * 16 + col + 1) * log2lam);  // L^(i + 1)
+        o[n][ti][0] *= w; o[n][ti][1] *= w; o[n][ti][2] *= w; o[n][ti][3] *= w;
+      }
+      // what the chunk's own tokens give
+      const uint16_t* v_row = v_t + (dt_e * 16 + col) * RC_TSTR + 4 * grp;
+      const u32x2 v0 = *reinterpret_cast<const u32x2*>(v_row), v1 = *reinterpret_cast<const u32x2*>(v_row + 16);
+      const u32x4 vv = {v0[0], v0[1], v1[0], v1[1]};
+#pragma unroll
+      for (int ti = 0; ti < 2; ++ti) {
+        o[n][ti] = RC_MFMA(vv, p_hi[ti], o[n][ti]);
+        o[n][ti] = RC_MFMA(vv, p_lo[ti], o[n][ti]);
+      }
+    }
+
+    // ---- the state after the chunk: S = L^n S + Kw^T V
+    const float shrink = exp2f(static_cast<float>(n_tok) * log2lam);
+#pragma unroll
+    for (int n = 0; n < NVW; ++n) {
+      const int dt_e = wave + 4 * n;
+      if (dt_e >= n_vt) continue;
+      const u32x4 vb = *reinterpret_cast<const u32x4*>(v_t + (dt_e * 16 + col) * RC_TSTR + 8 * grp);
+#pragma unroll
+      for (int dt = 0; dt < ND; ++dt) {
+        const u32x4 kh = *reinterpret_cast<const u32x4*>(kw_hi + (dt * 16 + col) * RC_TSTR + 8 * grp);
+        const u32x4 kl = *reinterpret_cast<const u32x4*>(kw_lo + (dt * 16 + col) * RC_TSTR + 8 * grp);
+        floatx4 acc = s[dt][n];
+        acc[0] *= shrink; acc[1] *= shrink; acc[2] *= shrink; acc[3] *= shrink;
+        acc = RC_MFMA(kh, vb, acc);
+        s[dt][n] = RC_MFMA(kl, vb, acc);
+      }
+    }
+
+    // ---- every token's norm over all value elements, the gate, the store
+    float sq[2] = {0.f, 0.f};
+#pragma unroll
+    for (int n = 0; n < NVW; ++n)
+#pragma unroll
+      for (int ti = 0; ti < 2; ++ti)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) sq[ti] += o[n][ti][i] * o[n][ti][i];
+#pragma unroll
+    for (int ti = 0; ti < 2; ++ti) {
+      sq[ti] += __shfl_xor(sq[ti], 16, 64);
+      sq[ti] += __shfl_xor(sq[ti], 32, 64);
+      if (grp == 0) red[wave * 32 + ti * 16 + col] = sq[ti];
+    }
+    __syncthreads();  // also: every wave is done with the chunk's arrays
+#pragma unroll
+    for (int ti = 0; ti < 2; ++ti) {
+      const int tok = ti * 16 + col;
+      const float total = red[tok] + red[32 + tok] + red[64 + tok] + red[96 + tok];
+      const float inv = 1.0f / sqrtf(total / static_cast<float>(vdim) + eps);
+      if (tok >= n_tok) continue;
+      const bf16_t* g_row = proj + static_cast<size_t>(c0 + tok) * ld + g_off + head * vdim;
+      bf16_t* o_row = out + (static_cast<size_t>(c0 + tok) * heads + head) * vdim;
+#pragma unroll
+      for (int n = 0; n < NVW; ++n) {
+        const int e0 = (wave + 4 * n) * 16 + 4 * grp;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          if (e0 + i < vdim) {
+            const float g = to_float(g_row[e0 + i]);
+            o_row[e0 + i].bits = float_to_bf16_bits((o[n][ti][i] * inv) * (g / (1.0f + expf(-g))));
+          }
+        }
+      }
+    }
+    __syncthreads();  // red is read before the next chunk's waves write it again
+  }
+
+#pragma unroll
+  for (int n = 0; n < NVW; ++n) {
+    const int e = (wave + 4 * n) * 16 + col;
+#pragma unroll
+    for (int dt = 0; dt < ND; ++dt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (e < vdim) st[static_cast<size_t>(dt * 16 + 4 * grp + i) * vdim + e] = s[dt][n][i];
+  }
+}
+
+// Arguments as for the recurrent form (bfloat16 only): proj [tokens, ld] with q, k, v and the gate
+// at their offsets; out [tokens, heads * vdim]; state float [slots, heads, dim, vdim].  dim a
+// multiple of 32 up to 256, vdim up to 256, rot_dims even and at most dim.
+extern "C" int pylon_retention_chunked(void* out, const void* proj, long long ld, int q_off, int k_off, int v_off,
+                                       int g_off, float* state, const float* decay, const float* inv_freq,
+                                       int rot_dims, const int* positions, const int* row_start, const int* row_slots,
+                                       int rows, int heads, int dim, int vdim, float eps, float k_scale,
+                                       hipStream_t stream) {
+  PYLON_REQUIRE(rows >= 0 && heads > 0, "retention_chunked: bad sizes");
+  PYLON_REQUIRE(dim >= 32 && dim % 32 == 0 && dim <= 256, "retention_chunked: keys of a multiple of 32 up to 256 elements, got %d", dim);
+  PYLON_REQUIRE(vdim >= 1 && vdim <= 256, "retention_chunked: values of up to 256 elements, got %d", vdim);
+  PYLON_REQUIRE(rot_dims >= 0 && rot_dims % 2 == 0 && rot_dims <= dim && (dim - rot_dims) % 2 == 0,
+                "retention_chunked: rot_dims %d does not fit a head of %d", rot_dims, dim);
+  PYLON_REQUIRE(rot_dims == 0 || inv_freq != nullptr, "retention_chunked: a rotation needs its frequencies");
+  if (rows == 0) return 0;
+  const int vdim16 = (vdim + 15) & ~15;
+  const int nvw = (vdim16 / 16 + 3) / 4;
+  const size_t lds = 2 * (4 * static_cast<size_t>(RC_CHUNK) * (dim + 8) + 2 * static_cast<size_t>(dim) * RC_TSTR +
+                          static_cast<size_t>(vdim16) * RC_TSTR) + sizeof(float) * 128;
+  dim3 grid(rows, heads), block(256);
+#define GO(KS, NVW) \
+  do { \
+  if (lds > 48 * 1024) \
+    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&retention_chunked_kernel<KS, NVW>), \
+                              hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)); \
+  hipLaunchKernelGGL((retention_chunked_kernel<KS, NVW>), grid, block, lds, stream, (bf16_t*)out, \
+                     (const bf16_t*)proj, ld, q_off, k_off, v_off, g_off, state, decay, inv_freq, rot_dims, \
+                     positions, row_start, row_slots, heads, vdim, eps, k_scale); \
+  } while (0)
+#define PICK(KS)                    \
+  do {                              \
+    if (nvw <= 1) GO(KS, 1);        \
+    else if (nvw <= 2) GO(KS, 2);   \
+    else GO(KS, 4);                 \
+  } while (0)
+  switch (dim / 32) {
+    case 1: PICK(1); break;
+    case 2: PICK(2); break;
+    case 3: PICK(3); break;
+    case 4: PICK(4); break;
+    case 5: PICK(5); break;
+    case 6: PICK(6); break;
+    case 7: PICK(7); break;
+    default: PICK(8); break;
+  }
+#undef PICK
+#undef GO
+  PYLON_LAUNCHED("retention_chunked");
+}

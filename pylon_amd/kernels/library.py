@@ -32,10 +32,11 @@ _SIGNATURES = {
     "pylon_silu_gate": [P, I, P, I, I, I, P],
     "pylon_qkv_prepare": [P, P, P, P, I, L, P, P, F, P, I, P, P, I, I, I, I, I, P],
     "pylon_paged_attention": [P, P, P, P, I, P, I, P, P, I, I, I, I, I, I, F, I, L, P, P, I, I, I, P],
-    "pylon_attention_sink": [P, P, L, P, P, P, I, P, P, I, I, I, I, I, I, F, P, P, I, I, I, P, L, I, P],
+    "pylon_attention_sink": [P, P, L, P, P, P, I, P, P, I, I, I, I, I, I, F, P, I, I, I, P, L, I, P],
     "pylon_add_normed_rmsnorm": [P, I, P, P, I, I, L, P, F, P, I, P, I, I, F, P],
     "pylon_short_conv": [P, I, P, I, P, I, P, P, P, I, I, I, I, P],
     "pylon_retention_recurrent": [P, P, I, L, I, I, I, I, P, P, P, I, P, P, P, I, I, I, I, F, F, P],
+    "pylon_retention_chunked": [P, P, L, I, I, I, I, P, P, P, I, P, P, P, I, I, I, I, F, F, P],
     "pylon_kv_store": [P, P, P, I, L, I, I, P, I, I, I, I, P],
     "pylon_gated_act": [P, I, P, I, I, I, F, F, F, P],
     "pylon_scale": [P, L, F, P],

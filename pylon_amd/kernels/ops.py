@@ -257,20 +257,26 @@ def sink_cuts(tokens: int, n_heads: int, n_kv_heads: int, max_len: int, units: O
     256 keys of the longest request (``max_len`` may be an upper bound)."""
     units = units or _lib.compute_units()
     group = n_heads // n_kv_heads
-    groups = tokens * n_kv_heads * (-(-group // min(4, group)))
+    groups = tokens * n_kv_heads * (-(-group // 4))
     cuts = 1
     while cuts < 64 and groups * cuts * 2 <= 2 * units and max_len >= cuts * 2 * 256:
         cuts *= 2
     return cuts
 
 
+def bias_by_distance(rel: torch.Tensor, bucket: torch.Tensor) -> torch.Tensor:
+    """float32 ``[heads, n]``: ``rel[bucket[d], head]`` for every distance ``d`` the bucket table
+    lists: a learned bias table looked up once, for kernels that keep a head's biases in LDS."""
+    return rel.float().index_select(0, bucket.long()).t().contiguous()
+
+
 def attention_sink(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
                    tiles: Optional[torch.Tensor], positions: Optional[torch.Tensor], *, page_size: int, scale: float,
-                   rel: Optional[torch.Tensor], bucket: Optional[torch.Tensor], sink: bool,
-                   cuts: int = 1) -> torch.Tensor:
+                   bias: Optional[torch.Tensor], sink: bool, cuts: int = 1) -> torch.Tensor:
     """Causal attention with a bias by distance and a sink on the matrix cores: bfloat16 ``q``
     ``[tokens, heads, head_dim]`` (maybe a slice of wider rows), keys ``[pages, page_size, kv_heads,
     head_dim]``, values transposed inside their pages ``[pages, kv_heads, v_dim, page_size]``.
+    ``bias`` float32 ``[heads, n]``: what is added to the scaled score at distance ``min(i - j, n - 1)``.
     ``tiles`` int32 ``[n, 4]`` (first token, count <= 32, block-table row, first position); or None
     with ``positions``: every token a tile of its own on its own row of the table.  ``cuts``
     workgroups share the keys of a tile and a second kernel merges their float partial results."""
@@ -282,7 +288,7 @@ def attention_sink(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
     if v_cache.shape != (pages, n_kv_heads, v_dim, psize) or psize != page_size or hd != head_dim:
         raise KernelError("attention_sink: cache geometry does not match page_size/head_dim")
     if not attention_sink_ok(q.dtype, head_dim=head_dim, v_dim=v_dim, page_size=page_size,
-                             bucket_len=0 if bucket is None else bucket.numel()):
+                             bucket_len=0 if bias is None else bias.shape[-1]):
         raise KernelError("attention_sink does not take this geometry")
     if k_cache.dtype != q.dtype or v_cache.dtype != q.dtype or n_heads % n_kv_heads:
         raise KernelError("attention_sink: q and the caches differ in dtype, or the heads do not group")
@@ -290,8 +296,8 @@ def attention_sink(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
         raise KernelError("attention_sink: the heads of a q row must lie side by side")
     if pages * page_size >= 2 ** 31 or block_table.dim() != 2:
         raise KernelError("attention_sink: the cache is too large for int32 slots, or the table is not 2-D")
-    if (rel is None) != (bucket is None) or (rel is not None and (rel.dim() != 2 or rel.shape[1] != n_heads)):
-        raise KernelError("attention_sink: rel [rows, heads] and bucket go together")
+    if bias is not None and (bias.dim() != 2 or bias.shape[0] != n_heads):
+        raise KernelError("attention_sink: bias must be [heads, distances]")
     if tiles is not None:
         if tiles.dim() != 2 or tiles.shape[1] != 4:
             raise KernelError("attention_sink: tiles must be [n, 4]")
@@ -307,9 +313,8 @@ def attention_sink(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
     _lib.call("pylon_attention_sink", _dev(out, "out"), q.data_ptr(), q.stride(0) if tokens > 1 else n_heads * head_dim,
               _dev(k_cache, "k_cache"), _dev(v_cache, "v_cache"), _dev(block_table, "block_table", torch.int32),
               block_table.shape[1], _dev(tiles, "tiles", torch.int32), _dev(positions, "positions", torch.int32),
-              n_tiles, n_heads, n_kv_heads, head_dim, v_dim, page_size, float(scale), _dev(rel, "rel", torch.float32),
-              _dev(bucket, "bucket", torch.int32), 0 if bucket is None else bucket.numel(), 1 if sink else 0,
-              int(cuts), _dev(partial, "partial"), 0 if partial is None else partial.numel(), tokens, _stream())
+              n_tiles, n_heads, n_kv_heads, head_dim, v_dim, page_size, float(scale), _dev(bias, "bias", torch.float32),
+              0 if bias is None else bias.shape[1], 1 if sink else 0, int(cuts), _dev(partial, "partial"), 0 if partial is None else partial.numel(), tokens, _stream())
     return out
 
 
@@ -374,13 +379,21 @@ def short_conv(h: torch.Tensor, weight: torch.Tensor, state: Optional[torch.Tens
     return out
 
 
+def retention_chunked_ok(dtype: torch.dtype, *, dim: int, vdim: int, rot_dims: int) -> bool:
+    """Whether the matrix-core form of retention takes this geometry (else the recurrent form does)."""
+    return (dtype == torch.bfloat16 and dim % 32 == 0 and 32 <= dim <= 256 and 1 <= vdim <= 256
+            and rot_dims % 2 == 0 and (dim - rot_dims) % 2 == 0)
+
+
 def retention_recurrent(proj: torch.Tensor, state: torch.Tensor, decay: torch.Tensor,
                         inv_freq: Optional[torch.Tensor], positions: torch.Tensor, row_start: torch.Tensor,
                         row_slots: torch.Tensor, *, rows: int, heads: int, dim: int, vdim: int, rot_dims: int,
-                        eps: float, k_scale: float) -> torch.Tensor:
+                        eps: float, k_scale: float, chunked: bool = False) -> torch.Tensor:
     """Retention, token by token: ``proj`` ``[tokens, 2 heads dim + 2 heads vdim]`` holds q, k, v
     and the gate side by side; ``state`` (float32 ``[slots, heads, dim, vdim]``) is read and left
-    up to date.  Returns the gated, per-head normalised output ``[tokens, heads * vdim]``."""
+    up to date.  Returns the gated, per-head normalised output ``[tokens, heads * vdim]``.
+    ``chunked``: the matrix-core form for bfloat16 prompt portions, 32 tokens at a time (same
+    arguments, same state)."""
     if proj.dim() != 2 or proj.shape[1] != 2 * heads * dim + 2 * heads * vdim or proj.stride(1) != 1:
         raise KernelError("retention: the projection's rows must hold q, k, v and the gate")
     tokens = proj.shape[0]
@@ -395,6 +408,16 @@ def retention_recurrent(proj: torch.Tensor, state: torch.Tensor, decay: torch.Te
     if not proj.is_cuda:
         raise KernelError("proj must live on the GPU; there is no CPU path")
     out = torch.empty((tokens, heads * vdim), dtype=proj.dtype, device=proj.device)
+    if chunked:
+        if not retention_chunked_ok(proj.dtype, dim=dim, vdim=vdim, rot_dims=rot_dims):
+            raise KernelError("retention: the chunked form does not take this geometry")
+        _lib.call("pylon_retention_chunked", _dev(out, "out"), proj.data_ptr(), proj.stride(0), 0, heads * dim,
+                  2 * heads * dim, 2 * heads * dim + heads * vdim, _dev(state, "state", torch.float32),
+                  _dev(decay, "decay", torch.float32), _dev(inv_freq, "inv_freq", torch.float32), int(rot_dims),
+                  _dev(positions, "positions", torch.int32), _dev(row_start, "row_start", torch.int32),
+                  _dev(row_slots, "row_slots", torch.int32), rows, heads, dim, vdim, float(eps), float(k_scale),
+                  _stream())
+        return out
     _lib.call("pylon_retention_recurrent", _dev(out, "out"), proj.data_ptr(), dtype_code(proj.dtype), proj.stride(0),
               0, heads * dim, 2 * heads * dim, 2 * heads * dim + heads * vdim, _dev(state, "state", torch.float32),
               _dev(decay, "decay", torch.float32), _dev(inv_freq, "inv_freq", torch.float32), int(rot_dims),

@@ -172,6 +172,16 @@ class SinkAttention(Part):
         self.add_param("out", (spec.hidden_size, spec.n_heads * spec.v_head_dim), dtype, device)
         self.add_param("rel", (spec.bias_rows, spec.n_heads), torch.float32, device, role="vector")
         self.bucket = torch.tensor(distance_buckets(spec.bias_rows, spec.bias_far), dtype=torch.int32).to(device)
+        self._bias = None  # (version of rel, the table looked up by distance)
+
+    def bias_by_distance(self) -> torch.Tensor:
+        """``rel`` looked up for every distance once, [heads, distances]; made anew when the
+        parameter has been written since (a load, random weights drawn in place)."""
+        rel = self.params["rel"]
+        key = (rel.data_ptr(), rel._version)
+        if self._bias is None or self._bias[0] != key:
+            self._bias = (key, ops.bias_by_distance(rel, self.bucket))
+        return self._bias[1]
 
     def cache_requirement(self) -> KVRequirement:
         spec = self.spec
@@ -204,8 +214,8 @@ class SinkAttention(Part):
             tiles = None if ctx.decode_only else ctx.token_tiles(ops.SINK_TILE)
             cuts = ops.sink_cuts(tokens, spec.n_heads, spec.n_kv_heads, ctx.max_len) if ctx.decode_only else 1
             context = ops.attention_sink(q, cache.k, v_cache, cache.block_table, tiles, ctx.positions,
-                                         page_size=page_size, scale=spec.scale, rel=self.params["rel"],
-                                         bucket=self.bucket, sink=spec.sink, cuts=cuts)
+                                         page_size=page_size, scale=spec.scale, bias=self.bias_by_distance(),
+                                         sink=spec.sink, cuts=cuts)
         else:
             context = ops.paged_attention(
                 q, cache.k, v_cache, cache.block_table, ctx.tok_row, ctx.positions, page_size=page_size,

@@ -17,6 +17,9 @@ from .base import Part, StateRequirement
 from .registry import build_part, register_part
 
 
+CHUNKED_FROM = 4  # a step whose longest row brings at least this many tokens takes the chunked form
+
+
 class Retention(Part):
     def __init__(self, spec: RetentionSpec, *, dtype: torch.dtype, device) -> None:
         super().__init__()
@@ -45,10 +48,15 @@ class Retention(Part):
             raise ValueError("a retention layer cannot borrow another run's state")
         rotary = self.position.rotary()
         proj = ops.linear(h, self.params["qkvg"], out_dtype=self.dtype)
+        rot_dims = rotary[1] if rotary else 0
+        # prompt portions of a bfloat16 model run 32 tokens at a time on the matrix cores; steps of
+        # single tokens, float32 models and odd head sizes token by token
+        chunked = (not ctx.decode_only and ctx.max_count >= CHUNKED_FROM and ops.retention_chunked_ok(
+            self.dtype, dim=spec.head_dim, vdim=spec.v_head_dim, rot_dims=rot_dims))
         mixed = ops.retention_recurrent(
             proj, cache.state, self.decay, rotary[0] if rotary else None, ctx.positions, ctx.row_start,
             ctx.row_slots, rows=ctx.rows, heads=spec.n_heads, dim=spec.head_dim, vdim=spec.v_head_dim,
-            rot_dims=rotary[1] if rotary else 0, eps=spec.norm_eps, k_scale=spec.head_dim ** -0.5)
+            rot_dims=rot_dims, eps=spec.norm_eps, k_scale=spec.head_dim ** -0.5, chunked=chunked)
         return ops.linear_for_residual(mixed, self.params["out"], out_dtype=self.dtype)
 
 

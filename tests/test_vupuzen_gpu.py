@@ -142,6 +142,53 @@ def test_retention_in_portions_carries_its_state(ops, heads, dim, vdim, rot):
     assert float((state[1] - 9.0).abs().max()) == 0.0
 
 
+@pytest.mark.parametrize("heads, dim, vdim, rot", [(2, 32, 32, 32), (3, 64, 48, 16), (1, 128, 128, 128), (2, 96, 8, 0),
+                                                     (1, 256, 200, 64)])
+def test_retention_in_chunks_on_the_matrix_cores(ops, heads, dim, vdim, rot):
+    """bfloat16 portions of two requests side by side, of sizes that fill chunks, leave ragged
+    ones and mix with single tokens, from a state that is not zero, against the plain rule."""
+    rng = np.random.default_rng(heads * 31 + dim)
+    rnd = lambda a: torch.tensor(a).to(torch.bfloat16).to(torch.float64).numpy()
+    total = 150
+    decay = tuple(rng.uniform(0.9, 1.0, size=heads))
+    qk, vg = heads * dim, heads * vdim
+    first = {0: 700, 1: 0}
+    want, proj, start = {}, {}, {}
+    for r in (0, 1):
+        proj[r] = rnd(rng.normal(size=(total, 2 * qk + 2 * vg)))
+        split = lambda a, n: a.reshape(total, heads, n).transpose(1, 0, 2)
+        q, k = split(proj[r][:, :qk], dim), split(proj[r][:, qk: 2 * qk], dim)
+        v, g = split(proj[r][:, 2 * qk: 2 * qk + vg], vdim), proj[r][:, 2 * qk + vg:]
+        positions = np.arange(first[r], first[r] + total)
+        if rot:
+            q, k = plain.rotate_half_layout(q, positions, rot, 500.0), plain.rotate_half_layout(k, positions, rot, 500.0)
+        start[r] = rng.normal(size=(heads, dim, vdim)) * (1.0 if r == 0 else 0.0)
+        o, _end = plain.retention(q, k * dim ** -0.5, v, decay, 1e-4, state=start[r])
+        want[r] = o.transpose(1, 0, 2).reshape(total, vg) * plain.silu(g)
+    state = torch.zeros((3, heads, dim, vdim), device=DEV)
+    state[2] = torch.tensor(start[0], dtype=torch.float32)
+    inv_freq = None
+    if rot:
+        inv_freq = (1.0 / (torch.tensor(500.0) ** (torch.arange(0, rot, 2, dtype=torch.float32) / rot))).to(DEV)
+    slot, at, got = {0: 2, 1: 0}, {0: 0, 1: 0}, {0: [], 1: []}
+    dec = torch.tensor(decay, dtype=torch.float32, device=DEV)
+    for step in ({0: 64, 1: 5}, {0: 1, 1: 33}, {1: 32}, {0: 40, 1: 1}, {0: 45, 1: 79}):
+        rows = list(step)
+        x = torch.tensor(np.concatenate([proj[r][at[r]: at[r] + step[r]] for r in rows]), dtype=torch.bfloat16, device=DEV)
+        pos = np.concatenate([np.arange(first[r] + at[r], first[r] + at[r] + step[r]) for r in rows])
+        starts = np.concatenate([[0], np.cumsum([step[r] for r in rows])])
+        out = ops.retention_recurrent(x, state, dec, inv_freq, i32(pos), i32(starts), i32(slot[r] for r in rows),
+                                      rows=len(rows), heads=heads, dim=dim, vdim=vdim, rot_dims=rot, eps=1e-4,
+                                      k_scale=dim ** -0.5, chunked=True).float().cpu().numpy()
+        for i, r in enumerate(rows):
+            got[r].append(out[starts[i]: starts[i + 1]])
+            at[r] += step[r]
+    for r in (0, 1):
+        g = np.concatenate(got[r])
+        assert len(g) == total
+        assert np.abs(g - want[r]).max() < 1.5e-2 * np.abs(want[r]).max(), r  # the output's own bfloat16 rounding
+
+
 def paged(x, page, order, pages):
     """[T, G, d] -> cache [pages, page, G, d] with the sequence's blocks on the pages ``order``."""
     total, groups, d = x.shape
@@ -236,7 +283,8 @@ def test_sink_attention_on_the_matrix_cores(ops, dim, vdim, heads, groups, rows,
     tiles = [(a, min(32, count - a), 1, first + a) for a in range(0, count, 32)]
     tiles = i32(np.array(tiles[::-1]).reshape(-1)).view(-1, 4)  # heaviest first, as the step function orders them
     common = dict(page_size=page, scale=scale, rel=rel_t, bucket=bucket, sink=True)
-    got = ops.attention_sink(qv, kc, vt, table, tiles, None, **common).float().cpu().numpy()
+    fast = dict(page_size=page, scale=scale, bias=ops.bias_by_distance(rel_t, bucket), sink=True)
+    got = ops.attention_sink(qv, kc, vt, table, tiles, None, **fast).float().cpu().numpy()
     assert not np.isnan(got).any()
     assert np.abs(got - want[first:]).max() < 2e-2 * max(1.0, np.abs(want).max())
     assert np.abs(got[-1, 0] - v[3, 0]).max() < 0.2
@@ -249,7 +297,7 @@ def test_sink_attention_on_the_matrix_cores(ops, dim, vdim, heads, groups, rows,
     singles = torch.tensor(np.stack([q[n - 1] for n in lengths]), dtype=torch.bfloat16, device=DEV)
     for cuts in (1, 2, 8):  # the keys of a request shared between workgroups, merged by a second kernel
         got = ops.attention_sink(singles, kc, vt, table, None, i32([n - 1 for n in lengths]), cuts=cuts,
-                                 **common).float().cpu().numpy()
+                                 **fast).float().cpu().numpy()
         for r, n in enumerate(lengths):
             assert np.abs(got[r] - want[n - 1]).max() < 2e-2 * max(1.0, np.abs(want).max()), (n, cuts)
     assert ops.sink_cuts(8, 32, 8, 128, units=256) == 1 and ops.sink_cuts(8, 32, 8, 2048, units=256) == 8
