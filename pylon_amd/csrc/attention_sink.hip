@@ -309,21 +309,20 @@ __global__ void attention_sink_merge_kernel(bf16_t* __restrict__ out, const floa
   const int lane = threadIdx.x & 63;
   if (item >= items) return;
   const float* src = partial + static_cast<size_t>(item) * cuts * (2 + vdim);
-  float m = -INFINITY;
-  for (int c = 0; c < cuts; ++c) m = fmaxf(m, src[c * (2 + vdim)]);
-  float l = 0.f;
-  for (int c = 0; c < cuts; ++c) {
-    const float mc = src[c * (2 + vdim)];
-    if (mc != -INFINITY) l += src[c * (2 + vdim) + 1] * __expf(mc - m);
-  }
-  const float inv = 1.0f / l;
-  for (int d = lane; d < vdim; d += 64) {
+  // lane c takes cut c's maximum and sum (at most 64 cuts); the values come in a loop whose loads
+  // do not wait for one another
+  const float mc = lane < cuts ? src[lane * (2 + vdim)] : -INFINITY;
+  const float lc = lane < cuts ? src[lane * (2 + vdim) + 1] : 0.f;
+  const float m = wave_max(mc);
+  const float w = (mc == -INFINITY) ? 0.f : __expf(mc - m);
+  const float inv = 1.0f / wave_sum(lc * w);
+  for (int d0 = 0; d0 < vdim; d0 += 64) {  // every lane stays in the loop: its weight is read by the others
+    const int d = d0 + lane;
+    const bool mine = d < vdim;
     float acc = 0.f;
-    for (int c = 0; c < cuts; ++c) {
-      const float mc = src[c * (2 + vdim)];
-      if (mc != -INFINITY) acc += src[c * (2 + vdim) + 2 + d] * __expf(mc - m);
-    }
-    out[static_cast<size_t>(item) * vdim + d].bits = float_to_bf16_bits(acc * inv);
+#pragma unroll 8
+    for (int c = 0; c < cuts; ++c) acc = fmaf(mine ? src[c * (2 + vdim) + 2 + d] : 0.f, __shfl(w, c, 64), acc);
+    if (mine) out[static_cast<size_t>(item) * vdim + d].bits = float_to_bf16_bits(acc * inv);
   }
 }
 

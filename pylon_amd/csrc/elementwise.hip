@@ -433,12 +433,52 @@ __global__ void gated_act_kernel(TO* __restrict__ out, const TI* __restrict__ gu
   }
 }
 
+// bfloat16 rows whose length is a multiple of 8: eight elements (16 bytes) per thread.
+__global__ void gated_act_bf16x8_kernel(uint4* __restrict__ out, const uint4* __restrict__ gu, int chunks, size_t total,
+                                        float alpha, float offset, float limit) {
+  size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const size_t step = static_cast<size_t>(gridDim.x) * blockDim.x;
+  for (; i < total; i += step) {
+    const size_t t = i / chunks;
+    const size_t c = i - t * chunks;
+    const uint4 g = gu[t * 2 * chunks + c];
+    const uint4 u = gu[t * 2 * chunks + chunks + c];
+    const uint32_t gw[4] = {g.x, g.y, g.z, g.w}, uw[4] = {u.x, u.y, u.z, u.w};
+    uint32_t r[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      float gv[2] = {__uint_as_float(gw[j] << 16), __uint_as_float(gw[j] & 0xffff0000u)};
+      float uv[2] = {__uint_as_float(uw[j] << 16), __uint_as_float(uw[j] & 0xffff0000u)};
+      float a[2];
+#pragma unroll
+      for (int k = 0; k < 2; ++k) {
+        if (limit > 0.f) {
+          gv[k] = fminf(gv[k], limit);
+          uv[k] = fminf(fmaxf(uv[k], -limit), limit);
+        }
+        a[k] = (gv[k] / (1.0f + expf(-alpha * gv[k]))) * (uv[k] + offset);
+      }
+      r[j] = static_cast<uint32_t>(float_to_bf16_bits(a[0])) | (static_cast<uint32_t>(float_to_bf16_bits(a[1])) << 16);
+    }
+    out[i] = uint4{r[0], r[1], r[2], r[3]};
+  }
+}
+
 extern "C" int pylon_gated_act(void* out, int out_dtype, const void* gate_up, int in_dtype, int tokens, int inter,
                                float alpha, float offset, float limit, hipStream_t stream) {
   PYLON_REQUIRE(pylon_valid_dtype(in_dtype) && pylon_valid_dtype(out_dtype), "gated_act: unknown dtype");
   PYLON_REQUIRE(tokens >= 0 && inter > 0, "gated_act: bad sizes tokens=%d inter=%d", tokens, inter);
   const size_t total = static_cast<size_t>(tokens) * inter;
   if (total == 0) return 0;
+  if (in_dtype == PYLON_BF16 && out_dtype == PYLON_BF16 && inter % 8 == 0 &&
+      (reinterpret_cast<uintptr_t>(out) & 15) == 0 && (reinterpret_cast<uintptr_t>(gate_up) & 15) == 0) {
+    const size_t chunks_total = total / 8;
+    size_t nblocks = (chunks_total + 255) / 256;
+    if (nblocks > 65535u * 16u) nblocks = 65535u * 16u;
+    hipLaunchKernelGGL(gated_act_bf16x8_kernel, dim3((unsigned)nblocks), dim3(256), 0, stream, (uint4*)out,
+                       (const uint4*)gate_up, inter / 8, chunks_total, alpha, offset, limit);
+    PYLON_LAUNCHED("gated_act");
+  }
   size_t blocks = (total + 255) / 256;
   if (blocks > 65535u * 16u) blocks = 65535u * 16u;
   dim3 grid((unsigned)blocks), block(256);

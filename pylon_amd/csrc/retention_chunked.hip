@@ -5,7 +5,9 @@
 //   S'  = L^n S + sum_j L^(n-1-j) k_j v_j^T
 //
 // (q and k rotated by their positions, k scaled), then out_i = o_i / rms(o_i) * silu(g_i) as in
-// the recurrent form.  One workgroup of four waves per (row of the step, head) walks the row's
+// the recurrent form; a chunk's tokens are neighbours in their request, so a token's angle is the
+// chunk's first angle plus its steps, and the rotation of token i comes from one sine and cosine
+// per frequency and chunk and a table of the steps'.  One workgroup of four waves per (row of the step, head) walks the row's
 // chunks in order.  The state stays in float accumulators for the whole walk, every wave
 // owning the columns (value elements) of its tiles; everything else of a chunk is staged in LDS.
 // All products run as 16x16x32 bfloat16 instructions with float accumulation, and every float
@@ -58,6 +60,9 @@ __global__ __launch_bounds__(256) void retention_chunked_kernel(
   uint16_t* v_t = kw_lo + dim * RC_TSTR;        // [vdim16][RC_TSTR]: values, transposed
   const int vdim16 = (vdim + 15) & ~15;
   float* red = reinterpret_cast<float*>(v_t + vdim16 * RC_TSTR);  // [4][32]
+  float* step_c = red + 128;                    // [32][half]: cos and sin of i * frequency, i = 0..31
+  float* step_s = step_c + RC_CHUNK * (rot_dims / 2);
+  float* base_all = step_s + RC_CHUNK * (rot_dims / 2);  // [2][cos, sin][half]: of a chunk's first position, in turns
 
   const int row = blockIdx.x, head = blockIdx.y;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -68,6 +73,49 @@ __global__ __launch_bounds__(256) void retention_chunked_kernel(
   const float log2lam = log2f(lam);
   const int half = rot_dims / 2;
   const int n_vt = vdim16 / 16;
+
+  // A chunk's tokens are neighbours: the angle of token i is that of the chunk's first token plus
+  // i steps, so a chunk needs one sine and cosine per frequency and the table of the steps'.
+  for (int idx = tid; idx < RC_CHUNK * half; idx += 256) {
+    const int i = idx / half, pr = idx - i * half;
+    sincosf(static_cast<float>(i) * inv_freq[pr], &step_s[idx], &step_c[idx]);
+  }
+  const bool wide = rot_dims % 16 == 0 && vdim % 8 == 0 && ld % 8 == 0 && q_off % 8 == 0 && k_off % 8 == 0 &&
+                    v_off % 8 == 0;  // 16-byte loads of the projection
+  const int pos_begin = begin < end ? positions[begin] : 0;
+  if (tid < half) sincosf(static_cast<float>(pos_begin) * inv_freq[tid], &base_all[half + tid], &base_all[tid]);
+  // With 16-byte loads a chunk travels global -> registers -> LDS, and the registers of the next
+  // chunk are filled while this one is computed.
+  constexpr int QKI = (KS + 3) / 4;
+  u32x4 qk_raw[QKI][4], v_raw[NVW];
+  auto fetch = [&](int c0, int n_tok) {
+#pragma unroll
+    for (int it = 0; it < QKI; ++it) {
+      const int idx = tid + it * 256;
+      const int tok = idx % RC_CHUNK, pr0 = (idx / RC_CHUNK) * 8;  // neighbours in a wave take neighbouring tokens
+      const bool rotated = pr0 < half;
+      const int d0 = rotated ? pr0 : rot_dims + 2 * (pr0 - half);
+      const int d1 = rotated ? d0 + half : d0 + 8;
+#pragma unroll
+      for (int a = 0; a < 4; ++a) qk_raw[it][a] = u32x4{0u, 0u, 0u, 0u};
+      if (idx < RC_CHUNK * (dim / 16) && tok < n_tok) {
+        const bf16_t* pr_row = proj + static_cast<size_t>(c0 + tok) * ld + head * dim;
+        qk_raw[it][0] = *reinterpret_cast<const u32x4*>(pr_row + q_off + d0);
+        qk_raw[it][1] = *reinterpret_cast<const u32x4*>(pr_row + q_off + d1);
+        qk_raw[it][2] = *reinterpret_cast<const u32x4*>(pr_row + k_off + d0);
+        qk_raw[it][3] = *reinterpret_cast<const u32x4*>(pr_row + k_off + d1);
+      }
+    }
+#pragma unroll
+    for (int it = 0; it < NVW; ++it) {
+      const int idx = tid + it * 256;
+      const int tok = idx % RC_CHUNK, e0 = (idx / RC_CHUNK) * 8;
+      v_raw[it] = u32x4{0u, 0u, 0u, 0u};
+      if (idx < RC_CHUNK * (vdim16 / 8) && tok < n_tok && e0 < vdim)
+        v_raw[it] = *reinterpret_cast<const u32x4*>(proj + static_cast<size_t>(c0 + tok) * ld + v_off + head * vdim + e0);
+    }
+  };
+  if (wide && begin < end) fetch(begin, end - begin < RC_CHUNK ? end - begin : RC_CHUNK);
 
   // S[d tile][own value tile]: column = value element, rows = key elements 4 grp + i
   floatx4 s[ND][NVW];
@@ -84,6 +132,74 @@ __global__ __launch_bounds__(256) void retention_chunked_kernel(
   for (int c0 = begin; c0 < end; c0 += RC_CHUNK) {
     const int n_tok = end - c0 < RC_CHUNK ? end - c0 : RC_CHUNK;
     // ---- stage the chunk: rotated q and k as two terms, decayed keys transposed, values transposed
+    const int turn = ((c0 - begin) / RC_CHUNK) & 1;
+    const float* base_c = base_all + turn * rot_dims;
+    const float* base_s = base_c + half;
+    __syncthreads();  // the tables of this chunk's angles are written
+    if (wide) {
+      // a thread takes eight pairs of one token: elements d0..d0+7 with d0+half.. (rotated), or
+      // sixteen neighbours (not rotated)
+#pragma unroll
+      for (int it = 0; it < QKI; ++it) {
+        const int idx = tid + it * 256;
+        if (idx >= RC_CHUNK * (dim / 16)) break;
+        const int tok = idx % RC_CHUNK, pr0 = (idx / RC_CHUNK) * 8;  // neighbours in a wave take neighbouring tokens
+        const bool rotated = pr0 < half;
+        const int d0 = rotated ? pr0 : rot_dims + 2 * (pr0 - half);
+        const int d1 = rotated ? d0 + half : d0 + 8;
+        const u32x4* raw = qk_raw[it];
+        float x[4][8];
+#pragma unroll
+        for (int a = 0; a < 4; ++a)
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            x[a][e] = __uint_as_float((e & 1) ? (raw[a][e >> 1] & 0xffff0000u) : (raw[a][e >> 1] << 16));
+        if (rotated) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const float bc = base_c[pr0 + e], bs = base_s[pr0 + e];
+            const float rc = step_c[tok * half + pr0 + e], rs = step_s[tok * half + pr0 + e];
+            const float cs = bc * rc - bs * rs, sn = bs * rc + bc * rs;
+            const float qa = x[0][e] * cs - x[1][e] * sn, qb = x[1][e] * cs + x[0][e] * sn;
+            const float ka = x[2][e] * cs - x[3][e] * sn, kb = x[3][e] * cs + x[2][e] * sn;
+            x[0][e] = qa; x[1][e] = qb; x[2][e] = ka; x[3][e] = kb;
+          }
+        }
+        const float w = tok < n_tok ? exp2f(static_cast<float>(n_tok - 1 - tok) * log2lam) : 0.f;
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+          const int d = (a & 1) ? d1 : d0;
+          u32x4 hi, lo;
+#pragma unroll
+          for (int e = 0; e < 8; e += 2) {
+            const float sc = a >= 2 ? k_scale : 1.0f;
+            uint32_t h, l;
+            rc_split(x[a][e] * sc, x[a][e + 1] * sc, h, l);
+            hi[e >> 1] = h;
+            lo[e >> 1] = l;
+          }
+          uint16_t* dst_hi = (a >= 2 ? k_hi : q_hi) + tok * QSTR + d;
+          uint16_t* dst_lo = (a >= 2 ? k_lo : q_lo) + tok * QSTR + d;
+          *reinterpret_cast<u32x4*>(dst_hi) = hi;
+          *reinterpret_cast<u32x4*>(dst_lo) = lo;
+          if (a >= 2) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+              rc_split1(x[a][e] * k_scale * w, kw_hi[(d + e) * RC_TSTR + tok], kw_lo[(d + e) * RC_TSTR + tok]);
+          }
+        }
+      }
+#pragma unroll
+      for (int it = 0; it < NVW; ++it) {
+        const int idx = tid + it * 256;
+        if (idx >= RC_CHUNK * (vdim16 / 8)) break;
+        const int tok = idx % RC_CHUNK, e0 = (idx / RC_CHUNK) * 8;
+        const u32x4 raw = v_raw[it];
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          v_t[(e0 + e) * RC_TSTR + tok] = static_cast<uint16_t>((e & 1) ? (raw[e >> 1] >> 16) : (raw[e >> 1] & 0xffffu));
+      }
+    } else {
     for (int idx = tid; idx < RC_CHUNK * (dim / 2); idx += 256) {
       const int tok = idx / (dim / 2), pr = idx - tok * (dim / 2);
       int d0, d1;
@@ -96,9 +212,8 @@ __global__ __launch_bounds__(256) void retention_chunked_kernel(
         q0 = to_float(qr[d0]); q1 = to_float(qr[d1]);
         k0 = to_float(kr[d0]); k1 = to_float(kr[d1]);
         if (pr < half) {
-          const float angle = static_cast<float>(positions[c0 + tok]) * inv_freq[pr];
-          float sn, cs;
-          sincosf(angle, &sn, &cs);
+          const float bc = base_c[pr], bs = base_s[pr], rc = step_c[tok * half + pr], rs = step_s[tok * half + pr];
+          const float cs = bc * rc - bs * rs, sn = bs * rc + bc * rs;
           const float a = q0 * cs - q1 * sn, b = q1 * cs + q0 * sn;
           q0 = a; q1 = b;
           const float e = k0 * cs - k1 * sn, f = k1 * cs + k0 * sn;
@@ -121,7 +236,15 @@ __global__ __launch_bounds__(256) void retention_chunked_kernel(
       if (tok < n_tok && e < vdim) bits = proj[static_cast<size_t>(c0 + tok) * ld + v_off + head * vdim + e].bits;
       v_t[e * RC_TSTR + tok] = bits;
     }
+    }
     __syncthreads();
+    if (c0 + RC_CHUNK < end) {
+      if (wide) fetch(c0 + RC_CHUNK, end - c0 - RC_CHUNK < RC_CHUNK ? end - c0 - RC_CHUNK : RC_CHUNK);
+      // the next chunk's first angle (a row's tokens are neighbours: its position is this one's plus 32)
+      float* next = base_all + (turn ^ 1) * rot_dims;
+      if (tid < half)
+        sincosf(static_cast<float>(pos_begin + (c0 - begin) + RC_CHUNK) * inv_freq[tid], &next[half + tid], &next[tid]);
+    }
 
     // ---- decayed scores, transposed: rows = tokens j, columns = tokens i; p[ti] holds for token
     // i = 16 ti + col the tokens j = 4 grp + i' (first four) and 16 + 4 grp + i' (last four)
@@ -249,6 +372,32 @@ __global__ __launch_bounds__(256) void retention_chunked_kernel(
       if (tok >= n_tok) continue;
       const bf16_t* g_row = proj + static_cast<size_t>(c0 + tok) * ld + g_off + head * vdim;
       bf16_t* o_row = out + (static_cast<size_t>(c0 + tok) * heads + head) * vdim;
+      if (wide && g_off % 8 == 0) {
+        // four neighbouring value elements a lane: 8-byte loads of the gate, all sent for first
+        u32x2 graw[NVW];
+#pragma unroll
+        for (int n = 0; n < NVW; ++n) {
+          const int e0 = (wave + 4 * n) * 16 + 4 * grp;
+          graw[n] = u32x2{0u, 0u};
+          if (e0 < vdim) graw[n] = *reinterpret_cast<const u32x2*>(g_row + e0);
+        }
+#pragma unroll
+        for (int n = 0; n < NVW; ++n) {
+          const int e0 = (wave + 4 * n) * 16 + 4 * grp;
+          if (e0 >= vdim) continue;
+          float y[4];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float g = __uint_as_float((i & 1) ? (graw[n][i >> 1] & 0xffff0000u) : (graw[n][i >> 1] << 16));
+            y[i] = (o[n][ti][i] * inv) * (g / (1.0f + expf(-g)));
+          }
+          u32x2 packed;
+          packed[0] = static_cast<uint32_t>(float_to_bf16_bits(y[0])) | (static_cast<uint32_t>(float_to_bf16_bits(y[1])) << 16);
+          packed[1] = static_cast<uint32_t>(float_to_bf16_bits(y[2])) | (static_cast<uint32_t>(float_to_bf16_bits(y[3])) << 16);
+          *reinterpret_cast<u32x2*>(o_row + e0) = packed;
+        }
+        continue;
+      }
 #pragma unroll
       for (int n = 0; n < NVW; ++n) {
         const int e0 = (wave + 4 * n) * 16 + 4 * grp;
@@ -293,7 +442,7 @@ extern "C" int pylon_retention_chunked(void* out, const void* proj, long long ld
   const int vdim16 = (vdim + 15) & ~15;
   const int nvw = (vdim16 / 16 + 3) / 4;
   const size_t lds = 2 * (4 * static_cast<size_t>(RC_CHUNK) * (dim + 8) + 2 * static_cast<size_t>(dim) * RC_TSTR +
-                          static_cast<size_t>(vdim16) * RC_TSTR) + sizeof(float) * 128;
+                          static_cast<size_t>(vdim16) * RC_TSTR) + sizeof(float) * (128 + (RC_CHUNK + 2) * rot_dims);
   dim3 grid(rows, heads), block(256);
 #define GO(KS, NVW) \
   do { \

@@ -12,7 +12,7 @@
 // new one after it has read the old: no other thread touches that (row, channel).
 #include "common.h"
 
-#define CONV_TILE 64
+#define CONV_TILE 16
 #define CONV_MAX_TAPS 8
 
 template <typename TI, typename TW, typename TO>
@@ -51,10 +51,17 @@ __global__ void short_conv_kernel(TO* __restrict__ out, const TI* __restrict__ h
       else if (first_tile) win[j + 1] = old[keep - (begin - src)];
     }
   }
-  for (int t = a; t < b; ++t) {
+  // a tile's inputs are fetched before the first sum, so that their trips to memory overlap
+  float xs[CONV_TILE];
+#pragma unroll
+  for (int n = 0; n < CONV_TILE; ++n) xs[n] = (a + n < b) ? to_float(h[static_cast<size_t>(a + n) * width + c]) : 0.f;
+#pragma unroll
+  for (int n = 0; n < CONV_TILE; ++n) {
+    const int t = a + n;
+    if (t >= b) break;
 #pragma unroll
     for (int j = 0; j < CONV_MAX_TAPS - 1; ++j) win[j] = win[j + 1];
-    const float x = to_float(h[static_cast<size_t>(t) * width + c]);
+    const float x = xs[n];
 #pragma unroll
     for (int j = 0; j < CONV_MAX_TAPS; ++j)
       if (j == taps - 1) win[j] = x;

@@ -183,7 +183,7 @@ def with_tensor_shapes(cfg: VupuzenConfig, shapes: Mapping[str, Tuple[int, ...]]
     return VupuzenConfig(**{**cfg.__dict__, "bias_rows": tuple(rows)})
 
 
-DEFAULT_BIAS_ROWS = 32  # for a configuration that comes without tensors (random weights) and names none
+DEFAULT_BIAS_ROWS = 16  # for a configuration that comes without tensors (random weights) and names none
 
 
 def _bias_rows(cfg: VupuzenConfig, index: int) -> int:

@@ -25,7 +25,7 @@ def _mlp(ff, limit):
 _P_ATT = _attention(4, 2, 16, 24, 20)
 _P_RET = _retention(2, 24, 8, (0.9, 0.97), 8, 10000.0)
 VUPUZEN_P = {
-    "architecture": "Vupuzen", "vocab": 211, "width": 64, "canon": {"taps": 4}, "norm": {"eps": 1e-5},
+    "architecture": "Vupuzen", "vocab": 211, "width": 64, "canon": {"taps": 4}, "norm": {"eps": 2e-5},
     "logit_scale": 0.7, "bias_rows": [12, None, None, 12, None],
     "layers": [
         {"type": "attention", "mixer": _P_ATT, "mlp": _mlp(96, 1.0)},
@@ -49,11 +49,11 @@ VUPUZEN_Q = {
 }
 # R: heads of the sizes of the matrix-core kernels, long enough contexts for several blocks.
 VUPUZEN_R = {
-    "architecture": "Vupuzen", "vocab": 160, "width": 128, "canon": {"taps": 3}, "norm": {"eps": 1e-5},
-    "logit_scale": 0.5, "bias_rows": [None, 16],
+    "architecture": "Vupuzen", "vocab": 160, "width": 128, "canon": {"taps": 5}, "norm": {"eps": 3e-6},
+    "logit_scale": 0.25, "bias_rows": [None, 16],
     "layers": [
-        {"type": "retention", "mixer": _retention(2, 64, 64, (0.96, 0.999), 32, 10000.0), "mlp": _mlp(192, 1.5)},
-        {"type": "attention", "mixer": _attention(4, 2, 64, 64, 300), "mlp": _mlp(192, 1.5)},
+        {"type": "retention", "mixer": _retention(2, 64, 64, (0.96, 0.999), 32, 10000.0), "mlp": _mlp(192, 2.0)},
+        {"type": "attention", "mixer": _attention(4, 2, 64, 64, 300), "mlp": _mlp(192, 2.0)},
     ],
 }
 CONFIGS = {"P": VUPUZEN_P, "Q": VUPUZEN_Q, "R": VUPUZEN_R}
