@@ -42,12 +42,16 @@ __device__ __forceinline__ void rc_split1(float a, uint16_t& hi, uint16_t& lo) {
 #define RC_MFMA(a, b, c) __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0)
 
 // KS: slabs of 32 key elements (dim = 32 KS); NVW: tiles of 16 value elements per wave (vdim <= 64 NVW).
-template <int KS, int NVW>
+// MODE 0: a workgroup walks all chunks of its (row, head) in order.  MODE 1 and 2 take one chunk a
+// workgroup (blockIdx.z), for requests too few to fill the chip with one workgroup a head: MODE 1 leaves
+// what the chunk alone adds to the state, U_c = sum_j L^(n-1-j) k_j v_j^T, in `chunk_state`; a scan kernel
+// turns that into the state before every chunk; MODE 2 computes the chunk's outputs from it.
+template <int KS, int NVW, int MODE>
 __global__ __launch_bounds__(256) void retention_chunked_kernel(
     bf16_t* __restrict__ out, const bf16_t* __restrict__ proj, long long ld, int q_off, int k_off, int v_off, int g_off,
     float* state, const float* __restrict__ decay, const float* __restrict__ inv_freq, int rot_dims,
     const int* __restrict__ positions, const int* __restrict__ row_start, const int* __restrict__ row_slots,
-    int heads, int vdim, float eps, float k_scale) {
+    int heads, int vdim, float eps, float k_scale, float* __restrict__ chunk_state, int max_chunks) {
   constexpr int dim = 32 * KS, ND = 2 * KS;
   constexpr int QSTR = dim + 8;  // row of a [token][element] array in LDS
   extern __shared__ uint16_t rc_lds[];
@@ -67,8 +71,13 @@ __global__ __launch_bounds__(256) void retention_chunked_kernel(
   const int row = blockIdx.x, head = blockIdx.y;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int col = lane & 15, grp = lane >> 4;
-  const int begin = row_start[row], end = row_start[row + 1];
-  float* st = state + ((static_cast<size_t>(row_slots[row]) * heads + head) * dim) * vdim;
+  const int row_begin = row_start[row], row_end = row_start[row + 1];
+  // the tokens this workgroup takes: the whole row, or one chunk of it
+  const int begin = MODE == 0 ? row_begin : row_begin + static_cast<int>(blockIdx.z) * RC_CHUNK;
+  const int end = MODE == 0 ? row_end : (begin + RC_CHUNK < row_end ? begin + RC_CHUNK : row_end);
+  if (begin >= end) return;
+  float* st = MODE != 0 ? chunk_state + (((static_cast<size_t>(row) * heads + head) * max_chunks + blockIdx.z) * dim) * vdim :
+              state + ((static_cast<size_t>(row_slots[row]) * heads + head) * dim) * vdim;
   const float lam = decay[head];
   const float log2lam = log2f(lam);
   const int half = rot_dims / 2;
@@ -126,7 +135,7 @@ __global__ __launch_bounds__(256) void retention_chunked_kernel(
     for (int dt = 0; dt < ND; ++dt)
 #pragma unroll
       for (int i = 0; i < 4; ++i)
-        s[dt][n][i] = (e < vdim) ? st[static_cast<size_t>(dt * 16 + 4 * grp + i) * vdim + e] : 0.f;
+        s[dt][n][i] = (MODE != 1 && e < vdim) ? st[static_cast<size_t>(dt * 16 + 4 * grp + i) * vdim + e] : 0.f;
   }
 
   for (int c0 = begin; c0 < end; c0 += RC_CHUNK) {
@@ -246,6 +255,8 @@ __global__ __launch_bounds__(256) void retention_chunked_kernel(
         sincosf(static_cast<float>(pos_begin + (c0 - begin) + RC_CHUNK) * inv_freq[tid], &next[half + tid], &next[tid]);
     }
 
+    floatx4 o[NVW][2];
+    if (MODE != 1) {
     // ---- decayed scores, transposed: rows = tokens j, columns = tokens i; p[ti] holds for token
     // i = 16 ti + col the tokens j = 4 grp + i' (first four) and 16 + 4 grp + i' (last four)
     u32x4 p_hi[2], p_lo[2];
@@ -284,7 +295,6 @@ __global__ __launch_bounds__(256) void retention_chunked_kernel(
     }
 
     // ---- outputs, transposed: rows = value elements of the wave's tiles, columns = tokens
-    floatx4 o[NVW][2];
 #pragma unroll
     for (int n = 0; n < NVW; ++n) {
       const int dt_e = wave + 4 * n;
@@ -331,6 +341,8 @@ __global__ __launch_bounds__(256) void retention_chunked_kernel(
       }
     }
 
+    }
+    if (MODE != 2) {
     // ---- the state after the chunk: S = L^n S + Kw^T V
     const float shrink = exp2f(static_cast<float>(n_tok) * log2lam);
 #pragma unroll
@@ -349,6 +361,8 @@ __global__ __launch_bounds__(256) void retention_chunked_kernel(
       }
     }
 
+    }
+    if (MODE != 1) {
     // ---- every token's norm over all value elements, the gate, the store
     float sq[2] = {0.f, 0.f};
 #pragma unroll
@@ -410,6 +424,7 @@ __global__ __launch_bounds__(256) void retention_chunked_kernel(
         }
       }
     }
+    }
     __syncthreads();  // red is read before the next chunk's waves write it again
   }
 
@@ -420,8 +435,40 @@ __global__ __launch_bounds__(256) void retention_chunked_kernel(
     for (int dt = 0; dt < ND; ++dt)
 #pragma unroll
       for (int i = 0; i < 4; ++i)
-        if (e < vdim) st[static_cast<size_t>(dt * 16 + 4 * grp + i) * vdim + e] = s[dt][n][i];
+        if (MODE != 2 && e < vdim) st[static_cast<size_t>(dt * 16 + 4 * grp + i) * vdim + e] = s[dt][n][i];
   }
+}
+
+// The state before every chunk from what every chunk adds: chunk_state[.., c] holds U_c on entry and
+// S_c (the state before chunk c) on exit, S_(c+1) = L^n S_c + U_c; the request's state slot receives
+// the state after the last chunk.  One thread an element of the state; a chunk's loads do not wait
+// for the chunk before.
+__global__ void retention_scan_kernel(float* __restrict__ chunk_state, float* __restrict__ state,
+                                      const float* __restrict__ decay, const int* __restrict__ row_start,
+                                      const int* __restrict__ row_slots, int heads, int per_head, int max_chunks) {
+  const int row = blockIdx.x / heads, head = blockIdx.x - row * heads;
+  const int x = blockIdx.y * blockDim.x + threadIdx.x;
+  if (x >= per_head) return;
+  const int count = row_start[row + 1] - row_start[row];
+  const int n_chunks = (count + RC_CHUNK - 1) / RC_CHUNK;
+  float* cs = chunk_state + (static_cast<size_t>(row) * heads + head) * max_chunks * per_head + x;
+  float* st = state + (static_cast<size_t>(row_slots[row]) * heads + head) * per_head + x;
+  const float log2lam = log2f(decay[head]);
+  float sv = *st;
+  for (int c0 = 0; c0 < n_chunks; c0 += 8) {
+    float u[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) u[i] = (c0 + i < n_chunks) ? cs[static_cast<size_t>(c0 + i) * per_head] : 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      if (c0 + i >= n_chunks) break;
+      const int left = count - (c0 + i) * RC_CHUNK;
+      const float shrink = exp2f(static_cast<float>(left < RC_CHUNK ? left : RC_CHUNK) * log2lam);
+      cs[static_cast<size_t>(c0 + i) * per_head] = sv;
+      sv = fmaf(shrink, sv, u[i]);
+    }
+  }
+  *st = sv;
 }
 
 // Arguments as for the recurrent form (bfloat16 only): proj [tokens, ld] with q, k, v and the gate
@@ -431,6 +478,7 @@ extern "C" int pylon_retention_chunked(void* out, const void* proj, long long ld
                                        int g_off, float* state, const float* decay, const float* inv_freq,
                                        int rot_dims, const int* positions, const int* row_start, const int* row_slots,
                                        int rows, int heads, int dim, int vdim, float eps, float k_scale,
+                                       int max_count, float* chunk_state, long long chunk_floats,
                                        hipStream_t stream) {
   PYLON_REQUIRE(rows >= 0 && heads > 0, "retention_chunked: bad sizes");
   PYLON_REQUIRE(dim >= 32 && dim % 32 == 0 && dim <= 256, "retention_chunked: keys of a multiple of 32 up to 256 elements, got %d", dim);
@@ -443,15 +491,32 @@ extern "C" int pylon_retention_chunked(void* out, const void* proj, long long ld
   const int nvw = (vdim16 / 16 + 3) / 4;
   const size_t lds = 2 * (4 * static_cast<size_t>(RC_CHUNK) * (dim + 8) + 2 * static_cast<size_t>(dim) * RC_TSTR +
                           static_cast<size_t>(vdim16) * RC_TSTR) + sizeof(float) * (128 + (RC_CHUNK + 2) * rot_dims);
-  dim3 grid(rows, heads), block(256);
+  // chunk_state given: one workgroup a chunk, in three launches (contributions, scan, outputs)
+  const int max_chunks = (max_count + RC_CHUNK - 1) / RC_CHUNK;
+  PYLON_REQUIRE(chunk_state == nullptr ||
+                    (max_count >= 1 && chunk_floats >= static_cast<long long>(rows) * heads * max_chunks * dim * vdim),
+                "retention_chunked: the chunks' states need rows x heads x chunks x dim x vdim floats");
+  const int mode = chunk_state != nullptr ? 1 : 0;
+  dim3 grid(rows, heads, mode ? max_chunks : 1), block(256);
+#define LAUNCH(KS, NVW, MODE) \
+  do { \
+    if (lds > 48 * 1024) \
+      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&retention_chunked_kernel<KS, NVW, MODE>), \
+                                hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)); \
+    hipLaunchKernelGGL((retention_chunked_kernel<KS, NVW, MODE>), grid, block, lds, stream, (bf16_t*)out, \
+                       (const bf16_t*)proj, ld, q_off, k_off, v_off, g_off, state, decay, inv_freq, rot_dims, \
+                       positions, row_start, row_slots, heads, vdim, eps, k_scale, chunk_state, max_chunks); \
+  } while (0)
 #define GO(KS, NVW) \
   do { \
-  if (lds > 48 * 1024) \
-    (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&retention_chunked_kernel<KS, NVW>), \
-                              hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)); \
-  hipLaunchKernelGGL((retention_chunked_kernel<KS, NVW>), grid, block, lds, stream, (bf16_t*)out, \
-                     (const bf16_t*)proj, ld, q_off, k_off, v_off, g_off, state, decay, inv_freq, rot_dims, \
-                     positions, row_start, row_slots, heads, vdim, eps, k_scale); \
+    if (mode == 0) { \
+      LAUNCH(KS, NVW, 0); \
+    } else { \
+      LAUNCH(KS, NVW, 1); \
+      hipLaunchKernelGGL(retention_scan_kernel, dim3(rows * heads, (dim * vdim + 255) / 256), dim3(256), 0, stream, \
+                         chunk_state, state, decay, row_start, row_slots, heads, dim * vdim, max_chunks); \
+      LAUNCH(KS, NVW, 2); \
+    } \
   } while (0)
 #define PICK(KS)                    \
   do {                              \
@@ -471,5 +536,6 @@ extern "C" int pylon_retention_chunked(void* out, const void* proj, long long ld
   }
 #undef PICK
 #undef GO
+#undef LAUNCH
   PYLON_LAUNCHED("retention_chunked");
 }

@@ -36,7 +36,7 @@ _SIGNATURES = {
     "pylon_add_normed_rmsnorm": [P, I, P, P, I, I, L, P, F, P, I, P, I, I, F, P],
     "pylon_short_conv": [P, I, P, I, P, I, P, P, P, I, I, I, I, P],
     "pylon_retention_recurrent": [P, P, I, L, I, I, I, I, P, P, P, I, P, P, P, I, I, I, I, F, F, P],
-    "pylon_retention_chunked": [P, P, L, I, I, I, I, P, P, P, I, P, P, P, I, I, I, I, F, F, P],
+    "pylon_retention_chunked": [P, P, L, I, I, I, I, P, P, P, I, P, P, P, I, I, I, I, F, F, I, P, L, P],
     "pylon_kv_store": [P, P, P, I, L, I, I, P, I, I, I, I, P],
     "pylon_gated_act": [P, I, P, I, I, I, F, F, F, P],
     "pylon_scale": [P, L, F, P],

@@ -379,6 +379,21 @@ def short_conv(h: torch.Tensor, weight: torch.Tensor, state: Optional[torch.Tens
     return out
 
 
+RETENTION_CHUNK = 32
+RETENTION_PARALLEL_BYTES = 1 << 29  # the most memory the chunks' states may take
+
+
+def retention_chunk_parallel(rows: int, heads: int, dim: int, vdim: int, max_count: int,
+                             units: Optional[int] = None) -> bool:
+    """Whether chunked retention takes one workgroup a chunk: when one workgroup a (row, head) would
+    leave most compute units idle, the rows are long enough for the two extra launches to pay, and
+    the chunks' states (float32, ``dim x vdim`` a chunk and head) fit a bound."""
+    units = units or _lib.compute_units()
+    chunks = -(-max_count // RETENTION_CHUNK)
+    return (rows * heads * 2 <= units and chunks >= 4
+            and rows * heads * chunks * dim * vdim * 4 <= RETENTION_PARALLEL_BYTES)
+
+
 def retention_chunked_ok(dtype: torch.dtype, *, dim: int, vdim: int, rot_dims: int) -> bool:
     """Whether the matrix-core form of retention takes this geometry (else the recurrent form does)."""
     return (dtype == torch.bfloat16 and dim % 32 == 0 and 32 <= dim <= 256 and 1 <= vdim <= 256
@@ -388,12 +403,15 @@ def retention_chunked_ok(dtype: torch.dtype, *, dim: int, vdim: int, rot_dims: i
 def retention_recurrent(proj: torch.Tensor, state: torch.Tensor, decay: torch.Tensor,
                         inv_freq: Optional[torch.Tensor], positions: torch.Tensor, row_start: torch.Tensor,
                         row_slots: torch.Tensor, *, rows: int, heads: int, dim: int, vdim: int, rot_dims: int,
-                        eps: float, k_scale: float, chunked: bool = False) -> torch.Tensor:
+                        eps: float, k_scale: float, chunked: bool = False,
+                        max_count: Optional[int] = None) -> torch.Tensor:
     """Retention, token by token: ``proj`` ``[tokens, 2 heads dim + 2 heads vdim]`` holds q, k, v
     and the gate side by side; ``state`` (float32 ``[slots, heads, dim, vdim]``) is read and left
     up to date.  Returns the gated, per-head normalised output ``[tokens, heads * vdim]``.
     ``chunked``: the matrix-core form for bfloat16 prompt portions, 32 tokens at a time (same
-    arguments, same state)."""
+    arguments, same state).  With ``max_count`` (the most tokens a row brings) and few rows it
+    takes one workgroup a chunk instead of one a (row, head): what every chunk adds to the state,
+    a scan over the chunks, then every chunk's outputs (:func:`retention_chunk_parallel`)."""
     if proj.dim() != 2 or proj.shape[1] != 2 * heads * dim + 2 * heads * vdim or proj.stride(1) != 1:
         raise KernelError("retention: the projection's rows must hold q, k, v and the gate")
     tokens = proj.shape[0]
@@ -411,12 +429,17 @@ def retention_recurrent(proj: torch.Tensor, state: torch.Tensor, decay: torch.Te
     if chunked:
         if not retention_chunked_ok(proj.dtype, dim=dim, vdim=vdim, rot_dims=rot_dims):
             raise KernelError("retention: the chunked form does not take this geometry")
+        chunk_state = None
+        if max_count is not None and retention_chunk_parallel(rows, heads, dim, vdim, max_count):
+            chunks = -(-max_count // RETENTION_CHUNK)
+            chunk_state = torch.empty((rows * heads * chunks * dim * vdim,), dtype=torch.float32, device=proj.device)
         _lib.call("pylon_retention_chunked", _dev(out, "out"), proj.data_ptr(), proj.stride(0), 0, heads * dim,
                   2 * heads * dim, 2 * heads * dim + heads * vdim, _dev(state, "state", torch.float32),
                   _dev(decay, "decay", torch.float32), _dev(inv_freq, "inv_freq", torch.float32), int(rot_dims),
                   _dev(positions, "positions", torch.int32), _dev(row_start, "row_start", torch.int32),
                   _dev(row_slots, "row_slots", torch.int32), rows, heads, dim, vdim, float(eps), float(k_scale),
-                  _stream())
+                  int(max_count or 0), _dev(chunk_state, "chunk_state"),
+                  0 if chunk_state is None else chunk_state.numel(), _stream())
         return out
     _lib.call("pylon_retention_recurrent", _dev(out, "out"), proj.data_ptr(), dtype_code(proj.dtype), proj.stride(0),
               0, heads * dim, 2 * heads * dim, 2 * heads * dim + heads * vdim, _dev(state, "state", torch.float32),

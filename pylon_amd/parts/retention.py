@@ -56,7 +56,8 @@ class Retention(Part):
         mixed = ops.retention_recurrent(
             proj, cache.state, self.decay, rotary[0] if rotary else None, ctx.positions, ctx.row_start,
             ctx.row_slots, rows=ctx.rows, heads=spec.n_heads, dim=spec.head_dim, vdim=spec.v_head_dim,
-            rot_dims=rot_dims, eps=spec.norm_eps, k_scale=spec.head_dim ** -0.5, chunked=chunked)
+            rot_dims=rot_dims, eps=spec.norm_eps, k_scale=spec.head_dim ** -0.5, chunked=chunked,
+            max_count=ctx.max_count)
         return ops.linear_for_residual(mixed, self.params["out"], out_dtype=self.dtype)
 
 

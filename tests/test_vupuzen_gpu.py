@@ -142,9 +142,10 @@ def test_retention_in_portions_carries_its_state(ops, heads, dim, vdim, rot):
     assert float((state[1] - 9.0).abs().max()) == 0.0
 
 
+@pytest.mark.parametrize("parallel", [False, True])
 @pytest.mark.parametrize("heads, dim, vdim, rot", [(2, 32, 32, 32), (3, 64, 48, 16), (1, 128, 128, 128), (2, 96, 8, 0),
                                                      (1, 256, 200, 64)])
-def test_retention_in_chunks_on_the_matrix_cores(ops, heads, dim, vdim, rot):
+def test_retention_in_chunks_on_the_matrix_cores(ops, heads, dim, vdim, rot, parallel):
     """bfloat16 portions of two requests side by side, of sizes that fill chunks, leave ragged
     ones and mix with single tokens, from a state that is not zero, against the plain rule."""
     rng = np.random.default_rng(heads * 31 + dim)
@@ -172,14 +173,20 @@ def test_retention_in_chunks_on_the_matrix_cores(ops, heads, dim, vdim, rot):
         inv_freq = (1.0 / (torch.tensor(500.0) ** (torch.arange(0, rot, 2, dtype=torch.float32) / rot))).to(DEV)
     slot, at, got = {0: 2, 1: 0}, {0: 0, 1: 0}, {0: [], 1: []}
     dec = torch.tensor(decay, dtype=torch.float32, device=DEV)
-    for step in ({0: 64, 1: 5}, {0: 1, 1: 33}, {1: 32}, {0: 40, 1: 1}, {0: 45, 1: 79}):
+    assert ops.retention_chunk_parallel(1, 10, 128, 128, 2048, units=256) and not ops.retention_chunk_parallel(
+        1, 10, 128, 128, 64, units=256) and not ops.retention_chunk_parallel(16, 10, 128, 128, 2048, units=256)
+    plan = ({0: 64, 1: 5}, {0: 1, 1: 33}, {1: 32}, {0: 40, 1: 1}, {0: 45, 1: 79})
+    if parallel:  # rows of four chunks and more, beside a short one
+        plan = ({0: 130, 1: 5}, {0: 20, 1: 145})
+    for step in plan:
         rows = list(step)
         x = torch.tensor(np.concatenate([proj[r][at[r]: at[r] + step[r]] for r in rows]), dtype=torch.bfloat16, device=DEV)
         pos = np.concatenate([np.arange(first[r] + at[r], first[r] + at[r] + step[r]) for r in rows])
         starts = np.concatenate([[0], np.cumsum([step[r] for r in rows])])
         out = ops.retention_recurrent(x, state, dec, inv_freq, i32(pos), i32(starts), i32(slot[r] for r in rows),
                                       rows=len(rows), heads=heads, dim=dim, vdim=vdim, rot_dims=rot, eps=1e-4,
-                                      k_scale=dim ** -0.5, chunked=True).float().cpu().numpy()
+                                      k_scale=dim ** -0.5, chunked=True,
+                                      max_count=max(step.values()) if parallel else None).float().cpu().numpy()
         for i, r in enumerate(rows):
             got[r].append(out[starts[i]: starts[i + 1]])
             at[r] += step[r]
