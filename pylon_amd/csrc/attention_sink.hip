@@ -302,6 +302,194 @@ __global__ __launch_bounds__(256) void attention_sink_kernel(
   }
 }
 
+// A step of single tokens: one workgroup per (token, key/value head, cut of the keys).  The heads of
+// the group (at most 16) sit side by side in the query columns of one tile, all at the token's
+// position, so a block's scores for the whole group cost what one head's cost; the four waves take
+// every fourth block of the cut and fetch their operands themselves (no wave reads what another
+// fetched, so nothing is staged and nothing waits at a barrier); at the end the four waves' partial
+// results (maximum, sum, unnormalised output, all float) meet in LDS and are merged in the order of
+// the waves: into the output if the keys are not cut, else into the cut's partial result for the
+// merge kernel.
+template <int KS, int NV>
+__global__ __launch_bounds__(256) void attention_sink_decode_kernel(
+    bf16_t* __restrict__ out, const bf16_t* __restrict__ q, long long q_stride, const bf16_t* __restrict__ k_cache,
+    const bf16_t* __restrict__ v_cache, const int* __restrict__ block_table, int table_width,
+    const int* __restrict__ positions, int n_heads, int n_kv_heads, int dim, int vdim, int page_size, float scale,
+    const float* __restrict__ bias, int bucket_len, int sink, int cuts, float* __restrict__ partial) {
+  extern __shared__ float bias_lds[];  // [group][bucket_len]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int col = lane & 15, grp = lane >> 4;
+  const int group = n_heads / n_kv_heads;
+  int b = blockIdx.x;
+  const int cut = b % cuts;
+  b /= cuts;
+  const int kvh = b % n_kv_heads;
+  const int tok = b / n_kv_heads;
+  const int pos = positions[tok];
+  const int* table = block_table + static_cast<size_t>(tok) * table_width;
+  const int my_head = kvh * group + (col < group ? col : group - 1);  // columns past the group repeat its last head
+  if (bias != nullptr) {
+    for (int i = threadIdx.x; i < group * bucket_len; i += 256) {
+      const int h = i / bucket_len;
+      bias_lds[i] = bias[static_cast<size_t>(kvh * group + h) * bucket_len + (i - h * bucket_len)];
+    }
+  }
+  __syncthreads();
+  const float* tbl = bias_lds + (col < group ? col : group - 1) * bucket_len;
+  const float far_bias = bias != nullptr ? tbl[bucket_len - 1] : 0.f;
+
+  bf16x8 qf[KS];
+  {
+    const bf16_t* qr = q + static_cast<size_t>(tok) * q_stride + static_cast<size_t>(my_head) * dim;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int d = ks * 32 + grp * 8;
+      u32x4 raw = {0u, 0u, 0u, 0u};
+      if (d < dim) raw = *reinterpret_cast<const u32x4*>(qr + d);
+      qf[ks] = __builtin_bit_cast(bf16x8, raw);
+    }
+  }
+  floatx4 o[NV];
+#pragma unroll
+  for (int dt = 0; dt < NV; ++dt) o[dt] = floatx4{0.f, 0.f, 0.f, 0.f};
+  const bool first = sink && cut == 0 && wave == 0;  // the sink belongs to one partial result
+  float m_run = first ? 0.f : -INFINITY;
+  float l_run = (first && grp == 0) ? 1.f : 0.f;
+
+  const int n_blocks = pos / AS_BLOCK + 1;
+  const int per_cut = (n_blocks + cuts - 1) / cuts;
+  const int kb_begin = cut * per_cut * AS_BLOCK;
+  const int kb_end = (cut + 1) * per_cut < n_blocks ? (cut + 1) * per_cut * AS_BLOCK : n_blocks * AS_BLOCK;
+  for (int kb = kb_begin + wave * AS_BLOCK; kb < kb_end; kb += 4 * AS_BLOCK) {
+    const int page = table[kb / page_size];
+    const int in_page = kb % page_size;
+    floatx4 s[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const size_t slot = static_cast<size_t>(page) * page_size + in_page + t * 16 + col;
+      const bf16_t* kr = k_cache + (slot * n_kv_heads + kvh) * dim;
+      s[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const int d = ks * 32 + grp * 8;
+        u32x4 raw = {0u, 0u, 0u, 0u};
+        if (d < dim) raw = *reinterpret_cast<const u32x4*>(kr + d);
+        s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, raw), qf[ks], s[t], 0, 0, 0);
+      }
+    }
+    bf16x8 vf[NV];
+    const bool ragged = kb + AS_BLOCK - 1 > pos;
+#pragma unroll
+    for (int dt = 0; dt < NV; ++dt) {
+      const int d = dt * 16 + col;
+      u32x4 raw = {0u, 0u, 0u, 0u};
+      if (d < vdim) {
+        const bf16_t* vr = v_cache + ((static_cast<size_t>(page) * n_kv_heads + kvh) * vdim + d) * page_size +
+                           in_page + 4 * grp;
+        const u32x2 a0 = *reinterpret_cast<const u32x2*>(vr);
+        const u32x2 a1 = *reinterpret_cast<const u32x2*>(vr + 16);
+        raw = u32x4{a0[0], a0[1], a1[0], a1[1]};
+        if (ragged) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const int key = kb + (e >> 2) * 16 + 4 * grp + (e & 3);
+            if (key > pos) raw[e >> 1] &= (e & 1) ? 0x0000ffffu : 0xffff0000u;
+          }
+        }
+      }
+      vf[dt] = __builtin_bit_cast(bf16x8, raw);
+    }
+    float sc[8];
+    const bool all_far = bias == nullptr || pos - (kb + AS_BLOCK - 1) >= bucket_len - 1;
+    float top = m_run;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int key = kb + (e >> 2) * 16 + 4 * grp + (e & 3);
+      const int dist = pos - key;
+      float add = far_bias;
+      if (!all_far) {
+        int idx = dist < 0 ? 0 : dist;
+        idx = idx < bucket_len - 1 ? idx : bucket_len - 1;
+        add = tbl[idx];
+      }
+      const float v = fmaf(s[e >> 2][e & 3], scale, add);
+      sc[e] = dist >= 0 ? v : -INFINITY;
+      top = fmaxf(top, sc[e]);
+    }
+    top = fmaxf(top, __shfl_xor(top, 16, 64));
+    top = fmaxf(top, __shfl_xor(top, 32, 64));
+    const float corr = (top == -INFINITY || m_run == -INFINITY) ? (m_run == -INFINITY ? 0.f : 1.f) : __expf(m_run - top);
+    float p[8], sum = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      p[e] = (sc[e] == -INFINITY) ? 0.f : __expf(sc[e] - top);
+      sum += p[e];
+    }
+    l_run = l_run * corr + sum;
+    m_run = top;
+    u32x4 hi, lo;
+#pragma unroll
+    for (int e = 0; e < 8; e += 2) {
+      const uint32_t a = __float_as_uint(p[e]), c = __float_as_uint(p[e + 1]);
+      hi[e >> 1] = __builtin_amdgcn_perm(c, a, 0x07060302u);
+      const float ra = p[e] - __uint_as_float(a & 0xffff0000u), rc = p[e + 1] - __uint_as_float(c & 0xffff0000u);
+      lo[e >> 1] = __builtin_amdgcn_perm(__float_as_uint(rc), __float_as_uint(ra), 0x07060302u);
+    }
+    const bf16x8 p_hi = __builtin_bit_cast(bf16x8, hi), p_lo = __builtin_bit_cast(bf16x8, lo);
+#pragma unroll
+    for (int dt = 0; dt < NV; ++dt) {
+      floatx4 acc = o[dt];
+      acc[0] *= corr; acc[1] *= corr; acc[2] *= corr; acc[3] *= corr;
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], p_hi, acc, 0, 0, 0);
+      o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], p_lo, acc, 0, 0, 0);
+    }
+  }
+  float l = l_run;
+  l += __shfl_xor(l, 16, 64);
+  l += __shfl_xor(l, 32, 64);
+  float* mrg = bias_lds + (bias != nullptr ? group * bucket_len : 4);  // [4 waves][group][2 + vdim]
+  if (col < group) {
+    float* mine = mrg + (wave * group + col) * (2 + vdim);
+    if (grp == 0) {
+      mine[0] = m_run;
+      mine[1] = l;
+    }
+#pragma unroll
+    for (int dt = 0; dt < NV; ++dt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (dt * 16 + 4 * grp + i < vdim) mine[2 + dt * 16 + 4 * grp + i] = o[dt][i];
+  }
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < group * vdim; idx += 256) {
+    const int h = idx / vdim, d = idx - h * vdim;
+    const float* src = mrg + h * (2 + vdim);
+    const int stride = group * (2 + vdim);
+    float m = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) m = fmaxf(m, src[w * stride]);
+    float total = 0.f, acc = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const float mw = src[w * stride];
+      const float f = (mw == -INFINITY) ? 0.f : __expf(mw - m);
+      total = fmaf(src[w * stride + 1], f, total);
+      acc = fmaf(src[w * stride + 2 + d], f, acc);
+    }
+    const size_t item = static_cast<size_t>(tok) * n_heads + kvh * group + h;
+    if (cuts == 1) {
+      out[item * vdim + d].bits = float_to_bf16_bits(acc / total);
+    } else {
+      float* dst = partial + (item * cuts + cut) * (2 + vdim);
+      if (d == 0) {
+        dst[0] = m;
+        dst[1] = total;
+      }
+      dst[2 + d] = acc;
+    }
+  }
+}
+
 // One wave per (token, head): out = sum_c o_c e^(m_c - m) / sum_c l_c e^(m_c - m), cuts in order.
 __global__ void attention_sink_merge_kernel(bf16_t* __restrict__ out, const float* __restrict__ partial, int items,
                                             int cuts, int vdim) {
@@ -353,11 +541,52 @@ extern "C" int pylon_attention_sink(void* out, const void* q, long long q_stride
   PYLON_REQUIRE(bias == nullptr || (bucket_len >= 1 && bucket_len <= AS_MAX_BIAS),
                 "attention_sink: a bias by distance is a table of 1 to %d entries a head", AS_MAX_BIAS);
   PYLON_REQUIRE(cuts >= 1 && cuts <= 64, "attention_sink: 1 to 64 cuts, got %d", cuts);
-  PYLON_REQUIRE(cuts == 1 || (partial != nullptr &&
-                              partial_floats >= static_cast<long long>(tokens) * n_heads * cuts * (2 + vdim)),
+  const int group = n_heads / n_kv_heads;
+  // single tokens whose group of heads fits a tile's columns and whose bias tables fit LDS: the
+  // kernel with the heads side by side, four partial results a cut
+  const bool side_by_side = tiles == nullptr && group <= 16 &&
+                            (bias == nullptr || static_cast<long long>(group) * bucket_len * 4 <= 64 * 1024) &&
+                            (cuts == 1 || (partial != nullptr &&
+                                           partial_floats >= static_cast<long long>(tokens) * n_heads * cuts * (2 + vdim)));
+  PYLON_REQUIRE(side_by_side || cuts == 1 ||
+                    (partial != nullptr && partial_floats >= static_cast<long long>(tokens) * n_heads * cuts * (2 + vdim)),
                 "attention_sink: cut keys need room for their partial results");
   if (n_tiles == 0) return 0;
-  const int group = n_heads / n_kv_heads;
+  if (side_by_side) {
+    const long long wgs = static_cast<long long>(tokens) * n_kv_heads * cuts;
+    PYLON_REQUIRE(wgs < (1ll << 31), "attention_sink: too many workgroups for one launch");
+    const size_t lds_d = sizeof(float) * ((bias != nullptr ? group * bucket_len : 4) + 4 * group * (2 + vdim));
+    const int ks_d = (dim + 31) / 32, nv_d = (vdim + 15) / 16;
+#define GO_D(KS, NV)                                                                                                \
+  do {                                                                                                              \
+    if (lds_d > 48 * 1024)                                                                                          \
+      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_sink_decode_kernel<KS, NV>),                \
+                                hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_d));                \
+    hipLaunchKernelGGL((attention_sink_decode_kernel<KS, NV>), dim3(static_cast<unsigned>(wgs)), dim3(256), lds_d,    \
+                       stream, (bf16_t*)out, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache,           \
+                       block_table, table_width, positions, n_heads, n_kv_heads, dim, vdim, page_size, scale, bias,  \
+                       bias != nullptr ? bucket_len : 1, sink, cuts, partial);                                       \
+  } while (0)
+#define PICK_D(KS)                  \
+  do {                              \
+    if (nv_d <= 2) GO_D(KS, 2);     \
+    else if (nv_d <= 4) GO_D(KS, 4);\
+    else if (nv_d <= 8) GO_D(KS, 8);\
+    else GO_D(KS, 16);              \
+  } while (0)
+    if (ks_d <= 1) PICK_D(1);
+    else if (ks_d <= 2) PICK_D(2);
+    else if (ks_d <= 4) PICK_D(4);
+    else PICK_D(8);
+#undef PICK_D
+#undef GO_D
+    if (cuts > 1) {
+      const int items = tokens * n_heads;
+      hipLaunchKernelGGL(attention_sink_merge_kernel, dim3((items + 3) / 4), dim3(256), 0, stream, (bf16_t*)out,
+                         partial, items, cuts, vdim);
+    }
+    PYLON_LAUNCHED("attention_sink");
+  }
   const int waves = 4;
   const int chunks = (group + waves - 1) / waves;
   const long long blocks = static_cast<long long>(n_tiles) * n_kv_heads * chunks * cuts;

@@ -10,7 +10,10 @@
 // of every sum depends on the row's length and the workgroup's size only.
 #include "common.h"
 
-template <typename TD, typename TO, int PER>
+// ND: the number of partial sums when it is one of the usual counts (all their loads are then sent for
+// before the first addition; a loop over a count only known at run time would wait for memory once
+// per partial sum), 0 for any other count.  The order of the additions is the same either way.
+template <typename TD, typename TO, int PER, int ND>
 __global__ void add_normed_rmsnorm_kernel(TO* __restrict__ out, float* resid, const TD* __restrict__ delta,
                                           int n_delta, long long delta_stride, const float* __restrict__ post_gain,
                                           float post_eps, const float* __restrict__ gain, int gain_stride,
@@ -25,15 +28,33 @@ __global__ void add_normed_rmsnorm_kernel(TO* __restrict__ out, float* resid, co
   if (dr) {
     float d[PER];
     float ss = 0.f;
+    if (ND > 0) {
+      float e[PER][ND > 0 ? ND : 1];
 #pragma unroll
-    for (int n = 0; n < PER; ++n) {
-      const int i = threadIdx.x + n * blockDim.x;
-      d[n] = 0.f;
-      if (i < dim) {
-        float v = to_float(dr[i]);
-        for (int p = 1; p < n_delta; ++p) v += to_float(dr[i + p * delta_stride]);
+      for (int n = 0; n < PER; ++n) {
+        const int i = threadIdx.x + n * blockDim.x;
+#pragma unroll
+        for (int p = 0; p < ND; ++p) e[n][p] = (i < dim) ? to_float(dr[i + p * delta_stride]) : 0.f;
+      }
+#pragma unroll
+      for (int n = 0; n < PER; ++n) {
+        float v = e[n][0];
+#pragma unroll
+        for (int p = 1; p < ND; ++p) v += e[n][p];
         d[n] = v;
         ss += v * v;
+      }
+    } else {
+#pragma unroll
+      for (int n = 0; n < PER; ++n) {
+        const int i = threadIdx.x + n * blockDim.x;
+        d[n] = 0.f;
+        if (i < dim) {
+          float v = to_float(dr[i]);
+          for (int p = 1; p < n_delta; ++p) v += to_float(dr[i + p * delta_stride]);
+          d[n] = v;
+          ss += v * v;
+        }
       }
     }
     float mult = 1.0f;
@@ -89,20 +110,29 @@ extern "C" int pylon_add_normed_rmsnorm(void* out, int out_dtype, float* resid, 
   const int threads = dim <= 256 ? 64 : (dim <= 2048 ? 256 : (dim <= 8192 ? 512 : 1024));
   const int per = (dim + threads - 1) / threads;
   dim3 grid(rows), block(threads);
-#define GO(TD, TO, PER)                                                                                         \
-  hipLaunchKernelGGL((add_normed_rmsnorm_kernel<TD, TO, PER>), grid, block, 0, stream, (TO*)out, resid,         \
+#define GO(TD, TO, PER, ND)                                                                                     \
+  hipLaunchKernelGGL((add_normed_rmsnorm_kernel<TD, TO, PER, ND>), grid, block, 0, stream, (TO*)out, resid,     \
                      (const TD*)delta, n_delta, delta_stride, post_gain, post_eps, gain, gain_stride, row_idx,  \
                      dim, eps, write_resid)
-#define PICK(TD, TO)            \
-  do {                          \
-    if (per <= 4) GO(TD, TO, 4);      \
-    else if (per <= 8) GO(TD, TO, 8); \
-    else GO(TD, TO, 16);        \
+#define PICK(TD, TO, ND)              \
+  do {                                \
+    if (per <= 4) GO(TD, TO, 4, ND);      \
+    else if (per <= 8) GO(TD, TO, 8, ND); \
+    else GO(TD, TO, 16, ND);          \
   } while (0)
-  if (delta_dtype == PYLON_F32 && out_dtype == PYLON_F32) PICK(float, float);
-  else if (delta_dtype == PYLON_F32) PICK(float, bf16_t);
-  else if (out_dtype == PYLON_F32) PICK(bf16_t, float);
-  else PICK(bf16_t, bf16_t);
+#define PARTS(TO)                                              \
+  do {                                                         \
+    if (n_delta == 1 || delta == nullptr) PICK(float, TO, 1);  \
+    else if (n_delta == 2) PICK(float, TO, 2);                 \
+    else if (n_delta == 4 && per <= 8) PICK(float, TO, 4);     \
+    else if (n_delta == 8 && per <= 8) PICK(float, TO, 8);     \
+    else PICK(float, TO, 0);                                   \
+  } while (0)
+  if (delta_dtype == PYLON_F32 && out_dtype == PYLON_F32) PARTS(float);
+  else if (delta_dtype == PYLON_F32) PARTS(bf16_t);
+  else if (out_dtype == PYLON_F32) PICK(bf16_t, float, 0);
+  else PICK(bf16_t, bf16_t, 0);
+#undef PARTS
 #undef PICK
 #undef GO
   PYLON_LAUNCHED("add_normed_rmsnorm");

@@ -297,13 +297,15 @@ class Runner:
                     raise ValueError(
                         f"The model supports at most {max_positions:,} tokens per request."
                     )
+        if self.graphs is not None and self.graphs.wants(entries):
+            # A replayed step cannot fail halfway: its pages are reserved before anything is launched,
+            # a capture runs no kernel, and the replay is one call.  So no state is copied for it.
+            logits = self.graphs.run(entries)
+            if logits is not None:
+                self.logit_slots = self.graphs.last_logit_slots
+                return logits
         saved = self.manager.snapshot_state([e.seq for e in entries])
         try:
-            if self.graphs is not None and self.graphs.wants(entries):
-                logits = self.graphs.run(entries)
-                if logits is not None:
-                    self.logit_slots = self.graphs.last_logit_slots
-                    return logits
             ctx = build_step(entries, self.manager, self.arena, vocab_size=self.model.spec.vocab_size,
                              chosen=self.chosen)
             self.logit_slots = ctx.logit_slots
