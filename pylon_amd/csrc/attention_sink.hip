@@ -18,7 +18,8 @@
 // that they carry sixteen bits of mantissa.  The sink is where the walk starts: maximum 0,
 // sum 1, output 0.  The waves of a workgroup take heads of one key/value head at the same
 // tokens: a block's keys and values are fetched once, with 16-byte loads of whole rows, into LDS
-// and read from there by every wave as operands (rows padded against bank conflicts).  Keys
+// (two buffers in turns: one barrier a block) and read from there by every wave as operands
+// (rows padded against bank conflicts).  Keys
 // may be cut over `cuts` workgroups, which then leave float partial results (maximum, sum,
 // unnormalised output) for a second small kernel to merge in order; the sink belongs to the
 // first cut.  The order of a query's sums depends on its position and the number of cuts only.
@@ -71,8 +72,9 @@ __global__ __launch_bounds__(256) void attention_sink_kernel(
   const int tstride = (bucket_len + 3) & ~3;  // keeps what follows the tables 16-byte aligned
   float* tbl = bias_lds + wave * tstride;
   const int kstr = dim + 8, vstr = AS_BLOCK + 4;  // LDS rows, padded
-  bf16_t* k_lds = reinterpret_cast<bf16_t*>(bias_lds + waves_per_group * tstride);
-  bf16_t* v_lds = k_lds + AS_BLOCK * kstr;
+  // two buffers of a block's keys and values, used in turns
+  bf16_t* kv_lds = reinterpret_cast<bf16_t*>(bias_lds + waves_per_group * tstride);
+  const int buf_elems = AS_BLOCK * kstr + ((vdim + 15) & ~15) * vstr;
   constexpr int threads = waves_per_group * 64;
   const float* bias_row = bias ? bias + static_cast<size_t>(head) * bucket_len : nullptr;
   if (bias != nullptr) {
@@ -140,7 +142,9 @@ __global__ __launch_bounds__(256) void attention_sink_kernel(
       }
     }
   };
-  auto stage = [&]() {
+  auto stage = [&](int turn) {
+    bf16_t* k_lds = kv_lds + turn * buf_elems;
+    bf16_t* v_lds = k_lds + AS_BLOCK * kstr;
 #pragma unroll
     for (int n = 0; n < KL; ++n) {
       const int c = threadIdx.x + n * threads;
@@ -159,12 +163,18 @@ __global__ __launch_bounds__(256) void attention_sink_kernel(
       }
     }
   };
-  if (kb_begin < kb_end) fetch(kb_begin);
-  for (int kb = kb_begin; kb < kb_end; kb += AS_BLOCK) {
-    __syncthreads();  // everybody has read the block before
-    stage();
-    __syncthreads();
-    if (kb + AS_BLOCK < kb_end) fetch(kb + AS_BLOCK);
+  // Block b is computed from one buffer while block b + 1, fetched during block b - 1's math, is
+  // written to the other and block b + 2 is sent for: one barrier a block.
+  if (kb_begin < kb_end) {
+    fetch(kb_begin);
+    stage(0);
+    if (kb_begin + AS_BLOCK < kb_end) fetch(kb_begin + AS_BLOCK);
+  }
+  __syncthreads();
+  int turn = 0;
+  for (int kb = kb_begin; kb < kb_end; kb += AS_BLOCK, turn ^= 1) {
+    const bf16_t* k_lds = kv_lds + turn * buf_elems;
+    const bf16_t* v_lds = k_lds + AS_BLOCK * kstr;
     // K operands: row = key, eight elements per lane and step
     floatx4 s[AS_QT][2];
 #pragma unroll
@@ -262,6 +272,11 @@ __global__ __launch_bounds__(256) void attention_sink_kernel(
         o[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], p_lo, acc, 0, 0, 0);
       }
     }
+    if (kb + AS_BLOCK < kb_end) {
+      stage(turn ^ 1);  // nobody reads that buffer: the block before this one is done everywhere
+      if (kb + 2 * AS_BLOCK < kb_end) fetch(kb + 2 * AS_BLOCK);
+    }
+    __syncthreads();
   }
 
 #pragma unroll
@@ -593,8 +608,9 @@ extern "C" int pylon_attention_sink(void* out, const void* q, long long q_stride
   PYLON_REQUIRE(blocks < (1ll << 31), "attention_sink: too many tiles for one launch");
   dim3 grid(static_cast<unsigned>(blocks)), block(64 * waves);
   const int table_len = bias != nullptr ? bucket_len : 1;
-  const size_t lds = sizeof(float) * waves * ((table_len + 3) & ~3) + 2 * (static_cast<size_t>(AS_BLOCK) * (dim + 8) +
-                                                              static_cast<size_t>((vdim + 15) / 16 * 16) * (AS_BLOCK + 4));
+  const size_t lds = sizeof(float) * waves * ((table_len + 3) & ~3) +
+                     2 * 2 * (static_cast<size_t>(AS_BLOCK) * (dim + 8) +
+                              static_cast<size_t>((vdim + 15) / 16 * 16) * (AS_BLOCK + 4));  // two buffers of bfloat16
   PYLON_REQUIRE(lds <= 160 * 1024, "attention_sink: the bias table and a block do not fit LDS");
   const int ks = (dim + 31) / 32, nv = (vdim + 15) / 16;
 #define GO(KS, NV) \

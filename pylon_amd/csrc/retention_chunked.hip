@@ -79,7 +79,7 @@ __global__ __launch_bounds__(256) void retention_chunked_kernel(
   float* st = MODE != 0 ? chunk_state + (((static_cast<size_t>(row) * heads + head) * max_chunks + blockIdx.z) * dim) * vdim :
               state + ((static_cast<size_t>(row_slots[row]) * heads + head) * dim) * vdim;
   const float lam = decay[head];
-  const float log2lam = log2f(lam);
+  const float log2lam = lam > 0.f ? log2f(lam) : -1e30f;  // a decay of zero: every power but the zeroth is zero
   const int half = rot_dims / 2;
   const int n_vt = vdim16 / 16;
 
@@ -453,7 +453,7 @@ __global__ void retention_scan_kernel(float* __restrict__ chunk_state, float* __
   const int n_chunks = (count + RC_CHUNK - 1) / RC_CHUNK;
   float* cs = chunk_state + (static_cast<size_t>(row) * heads + head) * max_chunks * per_head + x;
   float* st = state + (static_cast<size_t>(row_slots[row]) * heads + head) * per_head + x;
-  const float log2lam = log2f(decay[head]);
+  const float log2lam = decay[head] > 0.f ? log2f(decay[head]) : -1e30f;
   float sv = *st;
   for (int c0 = 0; c0 < n_chunks; c0 += 8) {
     float u[8];

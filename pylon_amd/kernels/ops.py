@@ -18,6 +18,11 @@ BF16 = 1
 _DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16}
 
 
+def compute_units() -> int:
+    """Compute units of the current device."""
+    return _lib.compute_units()
+
+
 def dtype_code(dtype: torch.dtype) -> int:
     try:
         return _DTYPE_CODE[dtype]
