@@ -149,15 +149,19 @@ def parse_config(data: Mapping) -> VupuzenConfig:
                 raise ValueError(f"{where}: unknown feed-forward kind {mlp['kind']!r} (known: dense)")
             mlp = MlpConfig("dense", _positive_int(mlp["ff"], "ff"), _positive(mlp["limit"], "limit"))
         shared = entry.get("weights_of")
-        layer = LayerConfig(entry["type"], _parse_mixer(entry["type"], entry["mixer"], where), mlp,
-                            None if shared is None else int(shared))
-        if shared is not None:
-            if not 0 <= layer.weights_of < index or layers[layer.weights_of].weights_of is not None:
-                raise ValueError(f"{where}: weights_of must name an earlier layer that has weights of its own")
-            first = layers[layer.weights_of]
-            if (first.type, first.mixer, first.mlp) != (layer.type, layer.mixer, layer.mlp):
-                raise ValueError(f"{where}: a layer that shares weights must equal the layer it shares them with")
-        layers.append(layer)
+        layers.append(LayerConfig(entry["type"], _parse_mixer(entry["type"], entry["mixer"], where), mlp,
+                                  None if shared is None else int(shared)))
+    for index, layer in enumerate(layers):
+        if layer.weights_of is None:
+            continue
+        where = f"layers[{index}]"
+        # the owner may stand before or behind the layer that borrows, but it owns its tensors itself
+        if not 0 <= layer.weights_of < len(layers) or layer.weights_of == index or \
+                layers[layer.weights_of].weights_of is not None:
+            raise ValueError(f"{where}: weights_of must name another layer that has weights of its own")
+        first = layers[layer.weights_of]
+        if (first.type, first.mixer, first.mlp) != (layer.type, layer.mixer, layer.mlp):
+            raise ValueError(f"{where}: a layer that shares weights must equal the layer it shares them with")
     if not layers:
         raise ValueError("the model has no layers")
     eos = data.get("eos_token_id")

@@ -22,6 +22,25 @@ def test_config_json_selects_the_architecture_and_round_trips():
     assert cfg.owner(3) == 0 and cfg.owner(4) == 1 and cfg.owner(2) == 2
 
 
+def test_a_layer_may_borrow_the_weights_of_a_later_layer():
+    from pylon_amd.config.registry import resolve
+
+    config = copy.deepcopy(VUPUZEN_P)
+    layers = config["layers"]
+    layers[0], layers[3] = layers[3], layers[0]  # the borrower first, its owner fourth
+    layers[0]["weights_of"] = 3
+    config["bias_rows"] = [None, None, None, 12, None]
+    arch = resolve(config)
+    cfg = arch.parse_config(config)
+    assert cfg.owner(0) == 3 and cfg.owner(3) == 3
+    spec = arch.model_spec(cfg)
+    assert [e.layer for e in spec.schedule] == [2, 0, 1, 2, 0] and len(spec.layers) == 3
+    assert spec.layers[2].mixer.bias_rows == 12
+    names = arch.weight_targets(cfg)
+    assert "l3.mix.rel" in names and "l0.mix.rel" not in names
+    assert names["l3.mix.q"].param == "layers.2.mixer.qkv"
+
+
 def test_layers_become_specs_and_a_schedule_that_reuses_weights():
     from pylon_amd.config.registry import resolve
 
