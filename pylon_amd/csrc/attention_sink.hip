@@ -8,8 +8,8 @@
 // values lie transposed inside every page, [page, kv head, vdim, slot in page], so that the
 // eight keys a lane feeds to a matrix instruction are neighbours in memory.
 //
-// A wavefront owns up to 32 consecutive tokens of one request and one query head, as two tiles
-// of 16 query columns.  It walks the keys in blocks of 32 (which never cross a page: pages are
+// A workgroup owns up to 32 consecutive tokens of one request and the (up to four) query heads of
+// one key/value head; each of its eight wavefronts one head and 16 of the tokens (one tile of query columns).  It walks the keys in blocks of 32 (which never cross a page: pages are
 // multiples of 32).  Scores are computed transposed, S^T = K Q^T (16x16x32 instructions: rows are
 // keys, columns are queries), so that everything that belongs to a query (its running maximum,
 // its sum, its output) lives in the lanes of that query's column, and the exponentials are
@@ -31,7 +31,7 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
 #define AS_BLOCK 32   // keys per step of the walk
-#define AS_QT 2       // query tiles of 16 per wave
+#define AS_QT 1       // query tiles of 16 per wave
 #define AS_MAX_BIAS 4096
 
 __device__ __forceinline__ uint32_t as_pack(float a, float b) {
@@ -40,15 +40,17 @@ __device__ __forceinline__ uint32_t as_pack(float a, float b) {
 
 // KS: steps of 32 key elements (dim <= 32 KS); NV: tiles of 16 value elements (vdim <= 16 NV).
 template <int KS, int NV>
-__global__ __launch_bounds__(256) void attention_sink_kernel(
+__global__ __launch_bounds__(512) void attention_sink_kernel(
     bf16_t* __restrict__ out, const bf16_t* __restrict__ q, long long q_stride, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, const int* __restrict__ block_table, int table_width,
     const int* __restrict__ tiles, const int* __restrict__ positions, int n_heads, int n_kv_heads, int dim, int vdim, int page_size, float scale,
     const float* __restrict__ bias, int bucket_len, int sink, int cuts, float* __restrict__ partial) {
+  // eight waves: wave & 3 names the head of the group, wave >> 2 which 16 of the tile's 32 tokens, so
+  // that every SIMD holds two waves that fill each other's waits
   constexpr int waves_per_group = 4;
-  constexpr int KL = (KS + 1) / 2, VL = (NV + 3) / 4;  // 16-byte pieces of a block a thread fetches
-  extern __shared__ float bias_lds[];  // [waves][bucket_len], then the block's keys and values
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  constexpr int KL = (KS + 3) / 4, VL = (NV + 7) / 8;  // 16-byte pieces of a block a thread fetches
+  extern __shared__ float bias_lds[];  // [heads of the workgroup][bucket_len], then the block's keys and values
+  const int lane = threadIdx.x & 63, wave = (threadIdx.x >> 6) & 3, qsel = threadIdx.x >> 8;
   const int col = lane & 15, grp = lane >> 4;
   const int group = n_heads / n_kv_heads;
   const int chunks = (group + waves_per_group - 1) / waves_per_group;
@@ -66,7 +68,7 @@ __global__ __launch_bounds__(256) void attention_sink_kernel(
   const int tok0 = tiles ? tiles[4 * tile] : tile, count = tiles ? tiles[4 * tile + 1] : 1;
   const int row = tiles ? tiles[4 * tile + 2] : tile, pos0 = tiles ? tiles[4 * tile + 3] : positions[tile];
   const int kv_last = pos0 + count - 1;
-  const int n_qt = count > 16 ? AS_QT : 1;  // a tile of up to 16 tokens (a single token, a portion's end) needs one
+  const int n_qt = (qsel == 0 || count > 16) ? 1 : 0;  // a tile of up to 16 tokens leaves the second half's waves idle
   const int* table = block_table + static_cast<size_t>(row) * table_width;
 
   const int tstride = (bucket_len + 3) & ~3;  // keeps what follows the tables 16-byte aligned
@@ -75,7 +77,7 @@ __global__ __launch_bounds__(256) void attention_sink_kernel(
   // two buffers of a block's keys and values, used in turns
   bf16_t* kv_lds = reinterpret_cast<bf16_t*>(bias_lds + waves_per_group * tstride);
   const int buf_elems = AS_BLOCK * kstr + ((vdim + 15) & ~15) * vstr;
-  constexpr int threads = waves_per_group * 64;
+  constexpr int threads = 2 * waves_per_group * 64;
   const float* bias_row = bias ? bias + static_cast<size_t>(head) * bucket_len : nullptr;
   if (bias != nullptr) {
 #pragma unroll 8
@@ -88,7 +90,7 @@ __global__ __launch_bounds__(256) void attention_sink_kernel(
   int qpos[AS_QT];
 #pragma unroll
   for (int qt = 0; qt < AS_QT; ++qt) {
-    const int qi = qt * 16 + col;
+    const int qi = (qt + qsel) * 16 + col;
     qpos[qt] = pos0 + qi;
     const int t = tok0 + (qi < count ? qi : count - 1);
     const bf16_t* qr = q + static_cast<size_t>(t) * q_stride + static_cast<size_t>(head) * dim;
@@ -284,7 +286,7 @@ __global__ __launch_bounds__(256) void attention_sink_kernel(
     float l = l_run[qt];
     l += __shfl_xor(l, 16, 64);
     l += __shfl_xor(l, 32, 64);
-    const int qi = qt * 16 + col;
+    const int qi = (qt + qsel) * 16 + col;
     if (qi >= count || idle) continue;
     if (cuts > 1) {
       // [token, head, cut, 2 + vdim]: maximum, sum, unnormalised output
@@ -606,7 +608,7 @@ extern "C" int pylon_attention_sink(void* out, const void* q, long long q_stride
   const int chunks = (group + waves - 1) / waves;
   const long long blocks = static_cast<long long>(n_tiles) * n_kv_heads * chunks * cuts;
   PYLON_REQUIRE(blocks < (1ll << 31), "attention_sink: too many tiles for one launch");
-  dim3 grid(static_cast<unsigned>(blocks)), block(64 * waves);
+  dim3 grid(static_cast<unsigned>(blocks)), block(2 * 64 * waves);
   const int table_len = bias != nullptr ? bucket_len : 1;
   const size_t lds = sizeof(float) * waves * ((table_len + 3) & ~3) +
                      2 * 2 * (static_cast<size_t>(AS_BLOCK) * (dim + 8) +

@@ -212,8 +212,8 @@ class SinkAttention(Part):
         q = qkv.as_strided((tokens, spec.n_heads, spec.head_dim), (qkv.stride(0), spec.head_dim, 1))
         if self._matrix_cores(page_size) and qkv.stride(0) % 8 == 0:
             # tiles heaviest first (turning every second run of the order round, as the plain prefill
-            # kernel's caller does, loses here: 227 -> 270 us at 2,048 tokens; the heaviest tile's own walk
-            # sets the time, and it should start first)
+            # kernel's caller does, loses here: 227 -> 270 us a layer at 2,048 tokens with four waves a
+            # workgroup, 5.81 -> 5.92 ms for eight layers with eight; the heaviest tile should start first)
             tiles = None if ctx.decode_only else ctx.token_tiles(ops.SINK_TILE)
             # a prompt portion's tiles keep their keys whole: cut in two or four, with the merge behind,
             # a 2,048-token prompt of eight layers took 6.18 and 6.58 ms against 5.82
