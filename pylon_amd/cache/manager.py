@@ -83,7 +83,7 @@ def plan_pool(budget_bytes: int, groups: Seq[object], *, page_size: int, max_req
     caps: List[Optional[int]] = []
     for group in groups:
         cap = full
-        if group.window is not None:
+        if group.window is not None:  # the most entries a token looks back over: a window, or a chunk
             own = (pages_for(group.window + chunk, page_size) + 1) * max_requests
             cap = own if cap is None else min(cap, own)
         caps.append(cap)
@@ -126,7 +126,9 @@ class KVGroup:
         # page, slot in page, key/value head, element.  Zero-filled so that a slot no
         # token has written yet holds finite numbers.
         self.k: Dict[int, torch.Tensor] = {c: torch.zeros(shape, dtype=dtype, device=device) for c in cache_ids}
-        self.v: Dict[int, torch.Tensor] = {c: torch.zeros(v_shape, dtype=dtype, device=device) for c in cache_ids}
+        # a group that keeps one entry per token only (``values`` False) has no second tensor
+        self.v: Dict[int, Optional[torch.Tensor]] = {
+            c: torch.zeros(v_shape, dtype=dtype, device=device) if requirement.values else None for c in cache_ids}
 
     def record_pages(self, slot: int, first_index: int, pages: List[int]) -> None:
         end = first_index + len(pages)
@@ -309,12 +311,12 @@ class CacheManager:
             seq.length += count
             seq._pending = None
             for group in self.groups:
-                window = group.requirement.window
-                if window is None:
+                if not group.requirement.bounded:
                     continue
                 # The next token sits at position `length`; it sees keys from
-                # length - window + 1 on.  A page whose last slot lies before that is dead.
-                first_needed = seq.length - window + 1
+                # length - window + 1 on (or from the start of its chunk).  A page whose last
+                # slot lies before that is dead.
+                first_needed = group.requirement.first_needed(seq.length)
                 pages = seq.pages[group.index]
                 dead = min(max(0, first_needed // self.page_size), len(pages))
                 for i in range(dead):

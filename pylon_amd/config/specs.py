@@ -22,6 +22,8 @@ class NormSpec:
     kind: str
     dim: int
     eps: float
+    # what is added to the stored weight before it multiplies: 1.0 for weights stored around zero
+    weight_offset: float = 0.0
 
 
 @dataclass(frozen=True)
@@ -37,6 +39,8 @@ class PositionSpec:
     theta: float = 10000.0
     rotary_dim: int = 0
     max_positions: int = 0
+    # True: element 2i turns together with its neighbour 2i + 1 instead of with i + rotary_dim/2
+    interleaved: bool = False
 
 
 @dataclass(frozen=True)
@@ -53,6 +57,13 @@ class AttentionSpec:
     qk_norm_eps: float = 1e-6
     window: Optional[int] = None  # None: every earlier key; w: the last w keys
     kind: str = "attention"
+    # "head": q and k are normed head by head, weights of head_dim elements; "projection": one
+    # norm over all heads of q at once and one over all heads of k, weights of the projections' sizes
+    qk_norm_over: str = "head"
+    v_head_dim: Optional[int] = None  # size of a value head where it differs from a key head's
+    # c: position i sees key j <= i only if floor(i / c) == floor(j / c), chunks counted from the
+    # request's first token (not together with a window)
+    chunk: Optional[int] = None
 
     @property
     def q_size(self) -> int:
@@ -61,6 +72,14 @@ class AttentionSpec:
     @property
     def kv_size(self) -> int:
         return self.n_kv_heads * self.head_dim
+
+    @property
+    def value_dim(self) -> int:
+        return self.head_dim if self.v_head_dim is None else self.v_head_dim
+
+    @property
+    def v_size(self) -> int:
+        return self.n_kv_heads * self.value_dim
 
 
 @dataclass(frozen=True)
@@ -83,6 +102,31 @@ class SinkAttentionSpec:
     sink: bool = True
     window: Optional[int] = None
     kind: str = "sink_attention"
+
+
+@dataclass(frozen=True)
+class LatentAttentionSpec:
+    """Softmax attention whose keys and values are made from one small latent per token, the only
+    thing cached: ``c = norm(W_dkv h)`` (``kv_rank`` numbers), per head ``k = W_uk c``,
+    ``v = W_uv c``; queries through a latent of their own, ``q = W_uq norm(W_dq h)``; no
+    positions; ``score = scale * q.k`` over a sliding ``window`` (None: every earlier key), a
+    ``chunk`` (as in :class:`AttentionSpec`) or everything before; with ``gate`` every head's
+    output is multiplied by ``sigmoid(W_g h)`` of that head before the output projection.  The
+    latents' norms divide by the root mean square (``norm_eps`` inside the root) and multiply by a
+    weight."""
+
+    hidden_size: int
+    n_heads: int
+    head_dim: int
+    v_head_dim: int
+    q_rank: int
+    kv_rank: int
+    scale: float
+    norm_eps: float
+    window: Optional[int] = None
+    chunk: Optional[int] = None
+    gate: bool = True
+    kind: str = "latent_attention"
 
 
 @dataclass(frozen=True)
@@ -124,6 +168,32 @@ class CappedGatedFeedForwardSpec:
     alpha: float = 1.702
     offset: float = 1.0
     kind: str = "capped_gated_mlp"
+
+
+@dataclass(frozen=True)
+class MixtureFeedForwardSpec:
+    """A mixture of ``n_experts`` gated feed-forwards of ``expert_size`` hidden units, of which
+    every token uses the ``top`` with the largest router logits ``W_r h + b`` (float32), weighted
+    by the softmax over those ``top`` logits alone; an expert is ``down(silu(gate(h)) * up(h))``.
+    With ``shared_size`` a further expert of that many hidden units runs for every token and is
+    added, multiplied by ``sigmoid(w_sg . h)`` if ``shared_gate``."""
+
+    hidden_size: int
+    n_experts: int
+    top: int
+    expert_size: int
+    shared_size: Optional[int] = None
+    shared_gate: bool = True
+    router_bias: bool = True
+    kind: str = "mixture"
+
+
+@dataclass(frozen=True)
+class LogitSoftcapSpec:
+    """``logits <- cap * tanh(logits / cap)``."""
+
+    cap: float
+    kind: str = "softcap"
 
 
 @dataclass(frozen=True)
@@ -181,6 +251,9 @@ class ScheduleEntry:
 
     layer: int
     cache: Optional[int] = None
+    # True: the embedded tokens (the stream as it was before the first run) are added to the
+    # stream once more right before this run
+    add_embedding: bool = False
 
 
 @dataclass(frozen=True)
@@ -222,3 +295,7 @@ class ModelSpec:
                 )
             out.append((entry.layer, cache, cache == index))
         return tuple(out)
+
+    def embedding_again(self) -> Tuple[bool, ...]:
+        """Per run: whether the embedded tokens are added to the stream before it."""
+        return tuple(entry.add_embedding for entry in self.schedule)

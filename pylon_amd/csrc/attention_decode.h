@@ -105,7 +105,7 @@ __global__ __launch_bounds__(AD_MAX_WAVES* PYLON_WAVE) void attention_decode_ker
   const int pos = positions[t];
 
   // the keys of this workgroup (all of them unless gridDim.z cuts them), then of this wave
-  const int first = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int first = first_visible(pos, window);  // a window, a chunk, or everything
   const int n_cuts = gridDim.z, cut = blockIdx.z;
   int per_cut = (pos + 1 - first + n_cuts - 1) / n_cuts;
   per_cut = (per_cut + AD_TILE - 1) / AD_TILE * AD_TILE;

@@ -40,7 +40,7 @@ static int check_decode_geometry(const char* name, int tokens, int n_heads, int 
                 AD_MAX_GROUP);
   PYLON_REQUIRE(head_dim == 64 || head_dim == 128 || head_dim == 256, "%s: head_dim %d is not 64, 128 or 256",
                 name, head_dim);
-  PYLON_REQUIRE(page_size > 0 && table_width > 0 && window >= 0, "%s: bad page size, width or window", name);
+  PYLON_REQUIRE(page_size > 0 && table_width > 0, "%s: bad page size or width", name);
   PYLON_REQUIRE(n_waves == 1 || n_waves == 2 || n_waves == 4 || n_waves == 8,
                 "%s: 1, 2, 4 or 8 waves per (token, head), got %d", name, n_waves);
   PYLON_REQUIRE(tokens <= 65535 && n_kv_heads <= 65535, "%s: too many tokens or heads for one launch", name);

@@ -1,6 +1,6 @@
 // Paged causal grouped-query attention, the exact and general form: any element type,
 // any head size up to 512 (multiples of 8 with 16-byte loads), any number of heads and groups,
-// any page size, optional sliding window.  One wavefront owns one (token, query head):
+// any page size, optional sliding window or chunks (first_visible in common.h).  One wavefront owns one (token, query head):
 // it walks that token's visible keys 64 at a time (one key per lane), keeps a running
 // maximum and sum in float, and accumulates the weighted values with one lane per
 // output element.  The walk starts at the first visible key of the token, so the order
@@ -75,7 +75,7 @@ __global__ void paged_attention_kernel(T* __restrict__ out, const T* __restrict_
   const int kvh = h / (n_heads / n_kv_heads);
   const int pos = positions[t];
   const int* table = block_table + static_cast<size_t>(tok_row[t]) * table_width;
-  const int first = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int first = first_visible(pos, window);
 
   float m = -INFINITY, l = 0.f;
   float acc[DIMS_PER_LANE];
@@ -170,7 +170,8 @@ static int launch_paged_attention(T* out, const T* q, const T* k_cache, const T*
 // rel: null, or float [rows, n_heads] with bucket: int [bucket_len], every entry a row of rel.
 // block_table: [rows, table_width] page ids; tok_row[t] names the table row of token t;
 // positions[t] is the token's index in its request; keys first(t)..positions[t] are read,
-// first(t) = max(0, positions[t] - window + 1) when window > 0, else 0.
+// first(t) = max(0, positions[t] - window + 1) when window > 0; the start of the token's chunk of
+// -window positions when window < 0; else 0.
 extern "C" int pylon_paged_attention(void* out, const void* q, const void* k_cache, const void* v_cache,
                                      int dtype, const int* block_table, int table_width,
                                      const int* tok_row, const int* positions, int tokens, int n_heads,
@@ -188,7 +189,6 @@ extern "C" int pylon_paged_attention(void* out, const void* q, const void* k_cac
   PYLON_REQUIRE(q_stride >= static_cast<long long>(n_heads) * head_dim, "paged_attention: q rows overlap");
   PYLON_REQUIRE(rel == nullptr || (bucket != nullptr && bucket_len >= 1),
                 "paged_attention: a bias by distance needs its table of buckets");
-  PYLON_REQUIRE(window >= 0, "paged_attention: window must be 0 (none) or positive");
   if (tokens == 0) return 0;
   PYLON_REQUIRE(static_cast<long long>(tokens) * n_heads / ATT_WAVES < (1ll << 31),
                 "paged_attention: too many (token, head) pairs for one launch");

@@ -76,7 +76,8 @@ __device__ __forceinline__ float softmax_prepare(floatx4 (&s)[AP_BK / 16], float
     // key kb + 16*kt + 4*grp + r is seen if it is at most qp and inside the window: compared
     // as 16*kt + r (a constant) against two numbers of this lane
     const int last_seen = qp - kb - 4 * grp;
-    const int first_seen = (window > 0) ? last_seen - window + 1 : -(1 << 30);
+    // a window (> 0), the query's chunk of -window positions (< 0), or everything
+    const int first_seen = (window != 0) ? first_visible(qp, window) - kb - 4 * grp : -(1 << 30);
 #pragma unroll
     for (int kt = 0; kt < AP_BK / 16; ++kt)
 #pragma unroll
@@ -186,7 +187,7 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
   const int tok0 = td[0], ntok = td[1], trow = td[2], pos0 = td[3];
   const int* table = block_table + static_cast<size_t>(trow) * table_width;
   const int kv_last = pos0 + ntok - 1;
-  const int k_lo = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
+  const int k_lo = first_visible(pos0, window);  // of the tile's first query, which sees furthest back
   const int kb_first = (k_lo / AP_BK) * AP_BK;
   // The request's page ids go to LDS once, so that finding a key's page costs no trip to
   // memory inside the loop (the host refuses requests with more pages than fit).
@@ -318,7 +319,7 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_kernel(
 
     // mask (only blocks that reach past the tile's first query, or a window's edge, need
     // it), running softmax, and the probabilities as row operands of the value product
-    const bool masked = kb + AP_BK - 1 > pos0 || window > 0;
+    const bool masked = kb + AP_BK - 1 > pos0 || window != 0;
     bf16x8 pa[QT][AP_BK / 32];
 #pragma unroll
     for (int qt = 0; qt < QT; ++qt) {
@@ -423,7 +424,7 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_direct_kernel(
   const int tok0 = td[0], ntok = td[1], trow = td[2], pos0 = td[3];
   const int* table = block_table + static_cast<size_t>(trow) * table_width;
   const int kv_last = pos0 + ntok - 1;
-  const int k_lo = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
+  const int k_lo = first_visible(pos0, window);  // of the tile's first query, which sees furthest back
   const int kb_first = (k_lo / AP_BK) * AP_BK;
 
   // A block of 64 keys lies inside one page.  Rows past the last key repeat it.
@@ -496,7 +497,7 @@ __global__ __launch_bounds__(256, 2) void attention_prefill_direct_kernel(
       vf[a][1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((AP_LDS(s16x4)*)(v_tile + v_at[a] + 16 * ROW)); \
     }                                                                                                  \
     __builtin_amdgcn_sched_barrier(0);                                                                 \
-    const bool masked = (KB) + AP_BK - 1 > pos0 || window > 0;                                         \
+    const bool masked = (KB) + AP_BK - 1 > pos0 || window != 0;                                         \
     bf16x8 pa[QT][AP_BK / 32];                                                                         \
     float shift[QT];                                                                                   \
     _Pragma("unroll") for (int qt = 0; qt < QT; ++qt) {                                                \
@@ -572,7 +573,7 @@ extern "C" int pylon_attention_prefill(void* out, const void* q, const void* k_c
                 rows);
   PYLON_REQUIRE(head_dim == 64 || head_dim == 128 || head_dim == 256,
                 "attention_prefill: head_dim %d is not 64, 128 or 256", head_dim);
-  PYLON_REQUIRE(page_size > 0 && table_width > 0 && window >= 0, "attention_prefill: bad page size, width or window");
+  PYLON_REQUIRE(page_size > 0 && table_width > 0, "attention_prefill: bad page size or width");
   PYLON_REQUIRE(table_width <= AP_TABLE, "attention_prefill: a request may hold at most %d pages, the table has %d columns",
                 AP_TABLE, table_width);
   PYLON_REQUIRE(static_cast<long long>(n_tiles) * n_kv_heads < (1LL << 31), "attention_prefill: too many tiles for one launch");

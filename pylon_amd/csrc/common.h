@@ -57,6 +57,16 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
+// The first key that a token at position pos sees, for the one integer by which the attention
+// kernels are told their mask: window > 0, the last `window` keys (itself included);
+// window < 0, the keys of its own chunk of -window positions, chunks counted from position 0;
+// 0, every key from the request's first on.
+__host__ __device__ __forceinline__ int first_visible(int pos, int window) {
+  if (window > 0) return pos - window + 1 > 0 ? pos - window + 1 : 0;
+  if (window < 0) return pos <= 0 ? 0 : pos / (-window) * (-window);
+  return 0;
+}
+
 // Sum over a workgroup of up to 1024 threads. `scratch` holds >= 16 floats of LDS.
 // Every thread gets the result; the order of additions depends only on blockDim.
 __device__ __forceinline__ float block_sum(float v, float* scratch) {

@@ -508,3 +508,20 @@ extern "C" int pylon_scale(float* x, long long count, float factor, hipStream_t 
   hipLaunchKernelGGL(scale_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, x, (size_t)count, factor);
   PYLON_LAUNCHED("scale");
 }
+
+// ---- soft cap in place: x <- cap * tanh(x / cap) ----------------------------------------------
+__global__ void softcap_kernel(float* __restrict__ x, size_t total, float cap) {
+  size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const size_t step = static_cast<size_t>(gridDim.x) * blockDim.x;
+  for (; i < total; i += step) x[i] = cap * tanhf(x[i] / cap);
+}
+
+extern "C" int pylon_softcap(float* x, long long count, float cap, hipStream_t stream) {
+  PYLON_REQUIRE(count >= 0, "softcap: negative count");
+  PYLON_REQUIRE(cap > 0.f, "softcap: the cap must be positive");
+  if (count == 0) return 0;
+  size_t blocks = (static_cast<size_t>(count) + 255) / 256;
+  if (blocks > 65535u * 16u) blocks = 65535u * 16u;
+  hipLaunchKernelGGL(softcap_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, x, (size_t)count, cap);
+  PYLON_LAUNCHED("softcap");
+}

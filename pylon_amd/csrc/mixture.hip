@@ -1,0 +1,258 @@
+// A mixture of gated feed-forward experts, token by token.
+//
+// route_top: from float router logits (a product computed elsewhere) plus a bias, the `top`
+//   experts with the largest logits (the lower index among equals) and the softmax over those
+//   logits alone; optionally sigmoid of one more logit per token, the gate of a shared expert.
+//   One wavefront per token, everything in float.
+// expert_gate_up: hidden[(t, s)] = silu(W_gate[e] x_t) * (W_up[e] x_t) for every token t and each of
+//   its chosen experts e = experts[t, s]; a workgroup takes one (token, choice) and some hidden
+//   units, the token's input in LDS, a wave a hidden unit at a time with the lanes along the row.
+// expert_down: out[t] = sum_s weight[t, s] W_down[e_s] hidden[(t, s)] (+ gate[t] * shared[t]), float.
+// Every sum runs over its row in one fixed order, so a token's result does not depend on what
+// else is in the batch.
+#include "common.h"
+
+#define MX_MAX_TOP 32
+
+__global__ void __launch_bounds__(256)
+route_top_kernel(int* __restrict__ experts, float* __restrict__ weights, float* __restrict__ shared_gate,
+                 const float* __restrict__ logits, long long row_stride, const float* __restrict__ bias,
+                 int tokens, int n_experts, int top) {
+  __shared__ float chosen[4][MX_MAX_TOP];
+  const int lane = threadIdx.x & (PYLON_WAVE - 1), wave = threadIdx.x / PYLON_WAVE;
+  const int t = blockIdx.x * 4 + wave;
+  if (t >= tokens) return;  // whole waves leave; no barrier follows
+  const float* row = logits + static_cast<size_t>(t) * row_stride;
+  // lane l keeps experts l, l + 64, ... (at most 8 of them)
+  float z[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int e = lane + PYLON_WAVE * i;
+    z[i] = e < n_experts ? row[e] + (bias != nullptr ? bias[e] : 0.f) : -INFINITY;
+  }
+  for (int k = 0; k < top; ++k) {
+    float best = -INFINITY;
+    int best_e = 0x7fffffff;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int e = lane + PYLON_WAVE * i;
+      if (e < n_experts && (z[i] > best || (z[i] == best && e < best_e)) && !(z[i] != z[i])) {
+        best = z[i];
+        best_e = e;
+      }
+    }
+#pragma unroll
+    for (int off = PYLON_WAVE / 2; off > 0; off >>= 1) {
+      const float other = __shfl_xor(best, off, PYLON_WAVE);
+      const int other_e = __shfl_xor(best_e, off, PYLON_WAVE);
+      if (other > best || (other == best && other_e < best_e)) {
+        best = other;
+        best_e = other_e;
+      }
+    }
+    if (best_e == 0x7fffffff) best_e = 0;  // nothing comparable left (NaN logits): expert 0
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      if (lane + PYLON_WAVE * i == best_e) z[i] = -INFINITY;  // taken; -inf also marks it for later rounds
+    if (lane == 0) {
+      experts[static_cast<size_t>(t) * top + k] = best_e;
+      chosen[wave][k] = best;
+    }
+    // an expert whose logit is -inf can be taken twice only if fewer than `top` finite logits exist
+  }
+  __builtin_amdgcn_wave_barrier();
+  if (lane == 0) {
+    const float m = chosen[wave][0];  // the largest: they were taken in falling order
+    float sum = 0.f;
+    for (int k = 0; k < top; ++k) {
+      const float p = expf(chosen[wave][k] - m);
+      chosen[wave][k] = p;
+      sum += p;
+    }
+    for (int k = 0; k < top; ++k) weights[static_cast<size_t>(t) * top + k] = chosen[wave][k] / sum;
+    if (shared_gate != nullptr) shared_gate[t] = 1.0f / (1.0f + expf(-row[n_experts]));
+  }
+}
+
+// logits: float [tokens, n_experts (+ 1 with shared_gate)], rows row_stride apart; bias: null or
+// float [n_experts]; experts int [tokens, top], weights float [tokens, top], shared_gate null or float [tokens].
+extern "C" int pylon_route_top(int* experts, float* weights, float* shared_gate, const float* logits,
+                               long long row_stride, const float* bias, int tokens, int n_experts, int top,
+                               hipStream_t stream) {
+  PYLON_REQUIRE(tokens >= 0 && n_experts >= 1 && n_experts <= 8 * PYLON_WAVE,
+                "route_top: 1 to %d experts, got %d", 8 * PYLON_WAVE, n_experts);
+  PYLON_REQUIRE(top >= 1 && top <= n_experts && top <= MX_MAX_TOP, "route_top: top %d of %d experts (at most %d)",
+                top, n_experts, MX_MAX_TOP);
+  PYLON_REQUIRE(row_stride >= n_experts + (shared_gate != nullptr ? 1 : 0), "route_top: rows of logits overlap");
+  if (tokens == 0) return 0;
+  hipLaunchKernelGGL(route_top_kernel, dim3((tokens + 3) / 4), dim3(256), 0, stream, experts, weights, shared_gate,
+                     logits, row_stride, bias, tokens, n_experts, top);
+  PYLON_LAUNCHED("route_top");
+}
+
+// The dot product of a weight row with a vector in LDS, the lanes of a wave along the row: every
+// lane returns its share (the caller adds the lanes up).  Rows of a multiple of 8 elements at
+// 16-byte aligned addresses are read 8 elements a lane and trip.
+template <typename T>
+__device__ __forceinline__ float row_dot_share(const T* __restrict__ row, const float* __restrict__ xs, int n,
+                                               int lane, bool wide);
+
+template <>
+__device__ __forceinline__ float row_dot_share<float>(const float* __restrict__ row, const float* __restrict__ xs,
+                                                      int n, int lane, bool wide) {
+  float acc = 0.f;
+  if (wide) {
+    for (int i = lane * 4; i < n; i += PYLON_WAVE * 4) {
+      const float4 w = *reinterpret_cast<const float4*>(row + i);
+      acc = fmaf(xs[i], w.x, acc);
+      acc = fmaf(xs[i + 1], w.y, acc);
+      acc = fmaf(xs[i + 2], w.z, acc);
+      acc = fmaf(xs[i + 3], w.w, acc);
+    }
+  } else {
+    for (int i = lane; i < n; i += PYLON_WAVE) acc = fmaf(xs[i], row[i], acc);
+  }
+  return acc;
+}
+
+template <>
+__device__ __forceinline__ float row_dot_share<bf16_t>(const bf16_t* __restrict__ row, const float* __restrict__ xs,
+                                                       int n, int lane, bool wide) {
+  float acc = 0.f;
+  if (wide) {
+    for (int i = lane * 8; i < n; i += PYLON_WAVE * 8) {
+      const uint4 raw = *reinterpret_cast<const uint4*>(row + i);
+      const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        acc = fmaf(xs[i + 2 * j], __uint_as_float(w[j] << 16), acc);
+        acc = fmaf(xs[i + 2 * j + 1], __uint_as_float(w[j] & 0xffff0000u), acc);
+      }
+    }
+  } else {
+    for (int i = lane; i < n; i += PYLON_WAVE) acc = fmaf(xs[i], to_float(row[i]), acc);
+  }
+  return acc;
+}
+
+template <typename TX, typename TW>
+__global__ void __launch_bounds__(256)
+expert_gate_up_kernel(TX* __restrict__ hidden, const TX* __restrict__ x, long long x_stride,
+                      const TW* __restrict__ w, long long w_stride, const int* __restrict__ experts, int top,
+                      int ff, int width, int units_per_block, int wide) {
+  extern __shared__ float xs[];  // the token's input
+  const int pair = blockIdx.y, t = pair / top;
+  const int lane = threadIdx.x & (PYLON_WAVE - 1), wave = threadIdx.x / PYLON_WAVE;
+  for (int i = threadIdx.x; i < width; i += 256) xs[i] = to_float(x[static_cast<size_t>(t) * x_stride + i]);
+  __syncthreads();
+  const int e = experts[pair];
+  const TW* gate = w + static_cast<size_t>(e) * 2 * ff * w_stride;
+  const TW* up = gate + static_cast<size_t>(ff) * w_stride;
+  const int j0 = blockIdx.x * units_per_block;
+  const int j1 = j0 + units_per_block < ff ? j0 + units_per_block : ff;
+  for (int j = j0 + wave; j < j1; j += 4) {
+    const float g = wave_sum(row_dot_share<TW>(gate + static_cast<size_t>(j) * w_stride, xs, width, lane, wide));
+    const float u = wave_sum(row_dot_share<TW>(up + static_cast<size_t>(j) * w_stride, xs, width, lane, wide));
+    if (lane == 0) hidden[static_cast<size_t>(pair) * ff + j] = from_float<TX>(g / (1.0f + expf(-g)) * u);
+  }
+}
+
+// x: [tokens, width] (rows x_stride apart); w: [n_experts, 2 ff, width] (rows w_stride apart), an
+// expert's gate rows then its up rows; experts: int [tokens, top]; hidden: [tokens * top, ff].
+extern "C" int pylon_expert_gate_up(void* hidden, const void* x, int x_dtype, long long x_stride, const void* w,
+                                    int w_dtype, long long w_stride, const int* experts, int tokens, int top, int ff,
+                                    int width, hipStream_t stream) {
+  PYLON_REQUIRE(pylon_valid_dtype(x_dtype) && pylon_valid_dtype(w_dtype), "expert_gate_up: unknown dtype");
+  PYLON_REQUIRE(!(x_dtype == PYLON_F32 && w_dtype == PYLON_BF16), "expert_gate_up: float inputs take float weights");
+  PYLON_REQUIRE(tokens >= 0 && top >= 1 && ff >= 1 && width >= 1, "expert_gate_up: sizes must be positive");
+  PYLON_REQUIRE(x_stride >= width && w_stride >= width, "expert_gate_up: rows overlap");
+  PYLON_REQUIRE(top <= MX_MAX_TOP, "expert_gate_up: at most %d experts a token", MX_MAX_TOP);
+  const size_t lds = sizeof(float) * width;
+  PYLON_REQUIRE(lds <= 64 * 1024, "expert_gate_up: a row of %d elements does not fit LDS", width);
+  if (tokens == 0) return 0;
+  const int per = w_dtype == PYLON_F32 ? 4 : 8;
+  const int wide = (width % per == 0 && w_stride % per == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0) ? 1 : 0;
+  const int units = 16;
+  // grid.y is limited to 65535: more pairs go in several launches of whole tokens
+  const long long pairs = static_cast<long long>(tokens) * top;
+  const long long per_launch = static_cast<long long>(65535 / top) * top;
+  for (long long first = 0; first < pairs; first += per_launch) {
+    const int n = static_cast<int>(pairs - first < per_launch ? pairs - first : per_launch);
+    dim3 grid((ff + units - 1) / units, n), block(256);
+    const size_t off = static_cast<size_t>(first);
+#define GO(TX, TW)                                                                                               \
+  hipLaunchKernelGGL((expert_gate_up_kernel<TX, TW>), grid, block, lds, stream, (TX*)hidden + off * ff,          \
+                     (const TX*)x + (off / top) * x_stride, x_stride, (const TW*)w, w_stride, experts + off, top, \
+                     ff, width, units, wide)
+    if (x_dtype == PYLON_F32) GO(float, float);
+    else if (w_dtype == PYLON_F32) GO(bf16_t, float);
+    else GO(bf16_t, bf16_t);
+#undef GO
+  }
+  PYLON_LAUNCHED("expert_gate_up");
+}
+
+template <typename TH, typename TW>
+__global__ void __launch_bounds__(256)
+expert_down_kernel(float* __restrict__ out, const TH* __restrict__ hidden, const TW* __restrict__ w,
+                   long long w_stride, const int* __restrict__ experts, const float* __restrict__ weights,
+                   const float* __restrict__ shared, const float* __restrict__ shared_gate, int top, int ff,
+                   int width, int cols_per_block, int wide) {
+  extern __shared__ float hs[];  // [top, ff]: the token's hidden activations of its chosen experts
+  const int t = blockIdx.y;
+  const int lane = threadIdx.x & (PYLON_WAVE - 1), wave = threadIdx.x / PYLON_WAVE;
+  for (int i = threadIdx.x; i < top * ff; i += 256) hs[i] = to_float(hidden[static_cast<size_t>(t) * top * ff + i]);
+  __syncthreads();
+  const int c0 = blockIdx.x * cols_per_block;
+  const int c1 = c0 + cols_per_block < width ? c0 + cols_per_block : width;
+  for (int c = c0 + wave; c < c1; c += 4) {
+    float acc = 0.f;
+    for (int s = 0; s < top; ++s) {
+      const int e = experts[static_cast<size_t>(t) * top + s];
+      const TW* row = w + (static_cast<size_t>(e) * width + c) * w_stride;
+      acc = fmaf(weights[static_cast<size_t>(t) * top + s], wave_sum(row_dot_share<TW>(row, hs + s * ff, ff, lane, wide)),
+                 acc);
+    }
+    if (lane == 0) {
+      if (shared != nullptr) {
+        const float g = shared_gate != nullptr ? shared_gate[t] : 1.f;
+        acc = fmaf(g, shared[static_cast<size_t>(t) * width + c], acc);
+      }
+      out[static_cast<size_t>(t) * width + c] = acc;
+    }
+  }
+}
+
+// hidden: [tokens * top, ff]; w: [n_experts, width, ff] (rows w_stride apart); experts int and
+// weights float [tokens, top]; shared: null or float [tokens, width], multiplied by shared_gate[t]
+// (null: by one) and added; out: float [tokens, width].
+extern "C" int pylon_expert_down(float* out, const void* hidden, int h_dtype, const void* w, int w_dtype,
+                                 long long w_stride, const int* experts, const float* weights, const float* shared,
+                                 const float* shared_gate, int tokens, int top, int ff, int width,
+                                 hipStream_t stream) {
+  PYLON_REQUIRE(pylon_valid_dtype(h_dtype) && pylon_valid_dtype(w_dtype), "expert_down: unknown dtype");
+  PYLON_REQUIRE(!(h_dtype == PYLON_F32 && w_dtype == PYLON_BF16), "expert_down: float inputs take float weights");
+  PYLON_REQUIRE(tokens >= 0 && top >= 1 && ff >= 1 && width >= 1, "expert_down: sizes must be positive");
+  PYLON_REQUIRE(w_stride >= ff, "expert_down: rows overlap");
+  const size_t lds = sizeof(float) * top * ff;
+  PYLON_REQUIRE(lds <= 64 * 1024, "expert_down: %d experts of %d hidden units do not fit LDS", top, ff);
+  if (tokens == 0) return 0;
+  const int per = w_dtype == PYLON_F32 ? 4 : 8;
+  const int wide = (ff % per == 0 && w_stride % per == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0) ? 1 : 0;
+  const int cols = 16;
+  for (int first = 0; first < tokens; first += 65535) {
+    const int n = tokens - first < 65535 ? tokens - first : 65535;
+    dim3 grid((width + cols - 1) / cols, n), block(256);
+    const size_t off = static_cast<size_t>(first);
+#define GO(TH, TW)                                                                                              \
+  hipLaunchKernelGGL((expert_down_kernel<TH, TW>), grid, block, lds, stream, out + off * width,                 \
+                     (const TH*)hidden + off * top * ff, (const TW*)w, w_stride, experts + off * top,           \
+                     weights + off * top, shared != nullptr ? shared + off * width : nullptr,                   \
+                     shared_gate != nullptr ? shared_gate + off : nullptr, top, ff, width, cols, wide)
+    if (h_dtype == PYLON_F32) GO(float, float);
+    else if (w_dtype == PYLON_F32) GO(bf16_t, float);
+    else GO(bf16_t, bf16_t);
+#undef GO
+  }
+  PYLON_LAUNCHED("expert_down");
+}

@@ -1,0 +1,128 @@
+// q/k/v preparation for attention whose norm runs over a whole projection: one norm over all
+// heads of q at once and one over all heads of k (each divided by the root mean square of the
+// whole row and multiplied by a weight of the row's size; either may be absent), then a rotation
+// of the first rot_dim elements of every head of q and k by position * inv_freq[i], pairing
+// either neighbours (2i, 2i + 1) or halves (i, i + rot_dim/2); q goes to q_out, k and v into the
+// token's cache slot.  Values may have another size than keys.  One workgroup per token; sums,
+// angles and rotation in float, one rounding at the end.
+#include "common.h"
+
+#define QW_THREADS 256
+
+template <typename T>
+__global__ void __launch_bounds__(QW_THREADS)
+qkv_prepare_wide_kernel(T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache,
+                        const T* __restrict__ qkv, long long row_stride, const float* __restrict__ q_weight,
+                        const float* __restrict__ k_weight, float eps, const float* __restrict__ inv_freq,
+                        int rot_dim, int interleaved, const int* __restrict__ positions,
+                        const int* __restrict__ slot_map, int n_heads, int n_kv_heads, int head_dim, int v_dim,
+                        int store) {
+  extern __shared__ float turn[];  // cos then sin of the token's rot_dim/2 angles
+  __shared__ float scratch[16];
+  const int t = blockIdx.x, tid = threadIdx.x;
+  const T* row = qkv + static_cast<size_t>(t) * row_stride;
+  const int q_size = n_heads * head_dim, k_size = n_kv_heads * head_dim, v_size = n_kv_heads * v_dim;
+  const int half = rot_dim / 2;
+  if (rot_dim > 0) {
+    const float pos = static_cast<float>(positions[t]);
+    for (int i = tid; i < half; i += QW_THREADS) {
+      float s, c;
+      sincosf(pos * inv_freq[i], &s, &c);
+      turn[i] = c;
+      turn[half + i] = s;
+    }
+  }
+  float inv_q = 1.f, inv_k = 1.f;
+  if (q_weight != nullptr) {
+    float sq = 0.f;
+    for (int e = tid; e < q_size; e += QW_THREADS) {
+      const float v = to_float(row[e]);
+      sq = fmaf(v, v, sq);
+    }
+    inv_q = 1.0f / sqrtf(block_sum(sq, scratch) / static_cast<float>(q_size) + eps);
+  }
+  if (store && k_weight != nullptr) {
+    float sq = 0.f;
+    for (int e = tid; e < k_size; e += QW_THREADS) {
+      const float v = to_float(row[q_size + e]);
+      sq = fmaf(v, v, sq);
+    }
+    inv_k = 1.0f / sqrtf(block_sum(sq, scratch) / static_cast<float>(k_size) + eps);
+  }
+  __syncthreads();  // the angles are in LDS
+
+  // one projection (q: part 0, k: part 1): norm, rotation, store
+  for (int part = 0; part < (store ? 2 : 1); ++part) {
+    const int size = part == 0 ? q_size : k_size;
+    const T* src = row + (part == 0 ? 0 : q_size);
+    const float* weight = part == 0 ? q_weight : k_weight;
+    const float inv = part == 0 ? inv_q : inv_k;
+    T* dst = part == 0 ? q_out + static_cast<size_t>(t) * q_size
+                       : k_cache + static_cast<size_t>(slot_map[t]) * k_size;
+    for (int e = tid; e < size; e += QW_THREADS) {
+      const int d = e % head_dim;
+      float x = to_float(src[e]) * inv * (weight != nullptr ? weight[e] : 1.f);
+      if (d < rot_dim) {
+        int i, other;
+        bool first;
+        if (interleaved) {
+          i = d >> 1;
+          first = (d & 1) == 0;
+          other = e - d + (d ^ 1);
+        } else {
+          first = d < half;
+          i = first ? d : d - half;
+          other = first ? e + half : e - half;
+        }
+        const float y = to_float(src[other]) * inv * (weight != nullptr ? weight[other] : 1.f);
+        const float c = turn[i], s = turn[half + i];
+        // the pair (u, v) becomes (u cos - v sin, v cos + u sin)
+        x = first ? x * c - y * s : x * c + y * s;
+      }
+      dst[e] = from_float<T>(x);
+    }
+  }
+  if (store) {
+    T* dst = v_cache + static_cast<size_t>(slot_map[t]) * v_size;
+    const T* src = row + q_size + k_size;
+    for (int e = tid; e < v_size; e += QW_THREADS) dst[e] = src[e];
+  }
+}
+
+// qkv: [tokens, n_heads*head_dim (+ n_kv_heads*head_dim + n_kv_heads*v_dim with store)], rows
+// row_stride elements apart.  q_out: [tokens, n_heads, head_dim].  k_cache: [slots, n_kv_heads,
+// head_dim], v_cache: [slots, n_kv_heads, v_dim], slot_map[t] the token's slot.  q_weight
+// [n_heads*head_dim] and k_weight [n_kv_heads*head_dim] float, or null for no norm.  inv_freq:
+// rot_dim/2 floats (rot_dim 0: no rotation); interleaved 1 pairs neighbours, 0 halves.
+extern "C" int pylon_qkv_prepare_wide(void* q_out, void* k_cache, void* v_cache, const void* qkv, int dtype,
+                                      long long row_stride, const float* q_weight, const float* k_weight, float eps,
+                                      const float* inv_freq, int rot_dim, int interleaved, const int* positions,
+                                      const int* slot_map, int tokens, int n_heads, int n_kv_heads, int head_dim,
+                                      int v_dim, int store, hipStream_t stream) {
+  PYLON_REQUIRE(pylon_valid_dtype(dtype), "qkv_prepare_wide: unknown dtype");
+  PYLON_REQUIRE(tokens >= 0 && n_heads > 0 && n_kv_heads > 0 && head_dim > 0 && v_dim > 0,
+                "qkv_prepare_wide: sizes must be positive");
+  PYLON_REQUIRE(rot_dim >= 0 && rot_dim % 2 == 0 && rot_dim <= head_dim,
+                "qkv_prepare_wide: rot_dim %d must be even and at most the head size %d", rot_dim, head_dim);
+  PYLON_REQUIRE(rot_dim == 0 || (inv_freq != nullptr && positions != nullptr),
+                "qkv_prepare_wide: a rotation needs frequencies and positions");
+  PYLON_REQUIRE(!store || (k_cache != nullptr && v_cache != nullptr && slot_map != nullptr),
+                "qkv_prepare_wide: storing needs the caches and the slot map");
+  const long long width = static_cast<long long>(n_heads) * head_dim +
+                          (store ? static_cast<long long>(n_kv_heads) * (head_dim + v_dim) : 0);
+  PYLON_REQUIRE(row_stride >= width, "qkv_prepare_wide: rows of %lld elements lie %lld apart", width, row_stride);
+  PYLON_REQUIRE(rot_dim * sizeof(float) <= 48 * 1024, "qkv_prepare_wide: rot_dim %d is too large", rot_dim);
+  if (tokens == 0) return 0;
+  const size_t lds = sizeof(float) * (rot_dim > 0 ? rot_dim : 1);
+  if (dtype == PYLON_F32)
+    hipLaunchKernelGGL((qkv_prepare_wide_kernel<float>), dim3(tokens), dim3(QW_THREADS), lds, stream, (float*)q_out,
+                       (float*)k_cache, (float*)v_cache, (const float*)qkv, row_stride, q_weight, k_weight, eps,
+                       inv_freq, rot_dim, interleaved, positions, slot_map, n_heads, n_kv_heads, head_dim, v_dim,
+                       store);
+  else
+    hipLaunchKernelGGL((qkv_prepare_wide_kernel<bf16_t>), dim3(tokens), dim3(QW_THREADS), lds, stream,
+                       (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache, (const bf16_t*)qkv, row_stride, q_weight,
+                       k_weight, eps, inv_freq, rot_dim, interleaved, positions, slot_map, n_heads, n_kv_heads,
+                       head_dim, v_dim, store);
+  PYLON_LAUNCHED("qkv_prepare_wide");
+}

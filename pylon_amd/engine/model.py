@@ -7,7 +7,9 @@ vocabulary head only at the tokens whose logits are wanted
 its layers goes into two optional lists of parts: "stream" parts between the embedding and
 the first layer (``forward(resid, ctx) -> resid``, the float32 residual stream of the step's
 tokens), "logits" parts after the head (``forward(logits, ctx) -> logits``, float32, one row
-per wanted token; under graph replay they must write in place).
+per wanted token; under graph replay they must write in place).  A schedule entry with
+``add_embedding`` has the embedded tokens (after the stream parts) added to the stream once more
+before its run: how a model that runs a stretch of layers several times feeds every further pass.
 """
 from __future__ import annotations
 
@@ -31,6 +33,7 @@ class Model(Part):
         self.dtype = dtype
         self.device = torch.device(device)
         self.schedule = spec.resolved_schedule()
+        self.embedding_again = spec.embedding_again()
         self.add_param("embed", (spec.vocab_size, spec.hidden_size), dtype, device)
         if not spec.tie_word_embeddings:
             self.add_param("lm_head", (spec.vocab_size, spec.hidden_size), dtype, device)
@@ -87,8 +90,12 @@ class Model(Part):
                           chosen=ctx.chosen)
         for part in self.stream_parts:
             resid = part.forward(resid, ctx)
+        # a schedule may add the embedded tokens to the stream again before some of its runs
+        embedded = resid.clone() if any(self.embedding_again) else None
         delta = None
-        for layer, cache_id, stores in self.schedule:
+        for (layer, cache_id, stores), again in zip(self.schedule, self.embedding_again):
+            if again:
+                ops.residual_add(resid, embedded)  # the pending output of the run before follows in the norm
             resid, delta = self.blocks[layer].forward(resid, delta, ctx, ctx.cache(cache_id), stores)
         if ctx.n_logits == 0:
             return None

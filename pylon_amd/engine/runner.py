@@ -331,7 +331,7 @@ def cache_needs(requirements: Seq[object], dtype: torch.dtype, max_requests: int
     groups = []
     for need, cache_ids in by_need.items():
         entry = _Bytes(len(cache_ids) * need.n_kv_heads * (need.head_dim + need.value_dim) * elem)
-        entry.window = need.window
+        entry.window = need.span
         groups.append(entry)
     state_bytes = sum(max_requests * math.prod(need.shape) * torch.empty((), dtype=need.dtype).element_size()
                       for need in states.values())

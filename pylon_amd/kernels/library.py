@@ -51,6 +51,14 @@ _SIGNATURES = {
     "pylon_argmax_static": [P, P, I, I, L, P, P, P],
     "pylon_probe_read": [P, L, P, P],
     "pylon_sample": [P, P, I, I, L, P, P, P, P, P, P],
+    "pylon_qkv_prepare_wide": [P, P, P, P, I, L, P, P, F, P, I, I, P, P, I, I, I, I, I, I, P],
+    "pylon_latent_prepare": [P, P, P, P, L, I, P, P, F, P, I, I, I, I, I, P],
+    "pylon_head_project": [P, P, I, L, P, I, P, I, I, I, I, P],
+    "pylon_gate_heads": [P, I, P, L, I, P],
+    "pylon_route_top": [P, P, P, P, L, P, I, I, I, P],
+    "pylon_expert_gate_up": [P, P, I, L, P, I, L, P, I, I, I, I, P],
+    "pylon_expert_down": [P, P, I, P, I, L, P, P, P, P, I, I, I, I, P],
+    "pylon_softcap": [P, L, F, P],
 }
 
 

@@ -190,13 +190,31 @@ def qkv_prepare(qkv: torch.Tensor, q_out: torch.Tensor, k_cache: Optional[torch.
               tokens, n_heads, n_kv_heads, head_dim, 1 if store_kv else 0, _stream())
 
 
+def mask_code(window: Optional[int], chunk: Optional[int] = None) -> int:
+    """The one integer by which the attention kernels are told which earlier keys a token sees:
+    ``w > 0`` the last ``w`` (itself included), ``-c < 0`` those of its own chunk of ``c``
+    positions (chunks counted from the request's first token), 0 all of them."""
+    if window is not None and chunk is not None:
+        raise KernelError("a mask is a window or chunks, not both")
+    if window is not None:
+        if window < 1:
+            raise KernelError("a window holds at least one key")
+        return int(window)
+    if chunk is not None:
+        if chunk < 1:
+            raise KernelError("a chunk holds at least one position")
+        return -int(chunk)
+    return 0
+
+
 def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                     block_table: torch.Tensor, tok_row: torch.Tensor, positions: torch.Tensor, *,
                     page_size: int, window: Optional[int], scale: float,
                     out: Optional[torch.Tensor] = None, rel: Optional[torch.Tensor] = None,
                     bucket: Optional[torch.Tensor] = None, sink: bool = False,
-                    v_transposed: bool = False) -> torch.Tensor:
-    """Causal attention of each token over its request's cached keys ``<=`` its position.
+                    v_transposed: bool = False, chunk: Optional[int] = None) -> torch.Tensor:
+    """Causal attention of each token over its request's cached keys ``<=`` its position (with
+    ``window`` the last so many, with ``chunk`` those of its own chunk: :func:`mask_code`).
     ``q`` is ``[tokens, heads, head_dim]`` and may be a slice of wider rows (a fused
     projection); values may have another size than keys.  ``rel`` (float32 ``[rows, heads]``)
     with ``bucket`` (int32 ``[n]``) adds ``rel[bucket[min(i - j, n - 1)], head]`` to the scaled
@@ -239,7 +257,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
               _dev(v_cache, "v_cache"), dtype_code(q.dtype), _dev(block_table, "block_table", torch.int32),
               block_table.shape[1], _dev(tok_row, "tok_row", torch.int32),
               _dev(positions, "positions", torch.int32), tokens, n_heads, n_kv_heads, head_dim,
-              page_size, int(window or 0), float(scale), v_dim, q.stride(0) if tokens > 1 else n_heads * head_dim,
+              page_size, mask_code(window, chunk), float(scale), v_dim, q.stride(0) if tokens > 1 else n_heads * head_dim,
               _dev(rel, "rel", torch.float32), _dev(bucket, "bucket", torch.int32),
               0 if bucket is None else bucket.numel(), 1 if sink else 0, 1 if v_transposed else 0, _stream())
     return out
@@ -495,6 +513,12 @@ def gated_act(gate_up: torch.Tensor, *, alpha: float, offset: float, limit: floa
     return out
 
 
+def softcap_(x: torch.Tensor, cap: float) -> torch.Tensor:
+    """``x <- cap * tanh(x / cap)`` in place (float32)."""
+    _lib.call("pylon_softcap", _dev(x, "x", torch.float32), x.numel(), float(cap), _stream())
+    return x
+
+
 def scale_(x: torch.Tensor, factor: float) -> torch.Tensor:
     """``x *= factor`` in place (float32)."""
     _lib.call("pylon_scale", _dev(x, "x", torch.float32), x.numel(), float(factor), _stream())
@@ -575,7 +599,8 @@ def _decode_scratch(tokens: int, n_heads: int, head_dim: int, n_cuts: int, devic
 def attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                      block_table: torch.Tensor, tok_row: Optional[torch.Tensor], positions: torch.Tensor, *,
                      page_size: int, window: Optional[int], scale: float, n_splits: int,
-                     n_cuts: int = 1, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                     n_cuts: int = 1, out: Optional[torch.Tensor] = None,
+                     chunk: Optional[int] = None) -> torch.Tensor:
     """Paged attention of a few bfloat16 query tokens; ``n_splits`` wavefronts share the
     keys of each (token, key/value head) and merge their partial results, after ``n_cuts``
     workgroups have shared them first (their partial results meet in a second small
@@ -603,7 +628,7 @@ def attention_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     _lib.call("pylon_attention_decode", _dev(out, "out"), _dev(q, "q"), _dev(k_cache, "k_cache"),
               _dev(v_cache, "v_cache"), _dev(block_table, "block_table", torch.int32), block_table.shape[1],
               _dev(tok_row, "tok_row", torch.int32), _dev(positions, "positions", torch.int32),
-              tokens, n_heads, n_kv_heads, head_dim, page_size, int(window or 0), float(scale),
+              tokens, n_heads, n_kv_heads, head_dim, page_size, mask_code(window, chunk), float(scale),
               int(n_splits), int(n_cuts), _dev(scratch, "scratch"), 0 if scratch is None else scratch.numel(),
               _stream())
     return out
@@ -706,7 +731,7 @@ def prefill_attention_ok(q: torch.Tensor, k_cache: torch.Tensor, block_table: Op
 def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                       block_table: torch.Tensor, tiles: torch.Tensor, *, page_size: int,
                       window: Optional[int], scale: float, rows: Optional[int] = None,
-                      out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                      out: Optional[torch.Tensor] = None, chunk: Optional[int] = None) -> torch.Tensor:
     """Paged causal attention of bfloat16 prompt portions on the matrix cores.  ``tiles`` is
     int32 ``[n, 4]``: first token index, token count, block-table row and first position of
     runs of at most ``rows // group`` consecutive tokens of one request; ``rows`` (64 or 128,
@@ -728,7 +753,7 @@ def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     _lib.call("pylon_attention_prefill", _dev(out, "out"), _dev(q, "q"), _dev(k_cache, "k_cache"),
               _dev(v_cache, "v_cache"), _dev(block_table, "block_table", torch.int32), block_table.shape[1],
               _dev(tiles, "tiles", torch.int32), tiles.shape[0], n_heads, n_kv_heads, head_dim, page_size,
-              int(window or 0), float(scale), int(rows), _stream())
+              mask_code(window, chunk), float(scale), int(rows), _stream())
     return out
 
 
@@ -989,6 +1014,174 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_p: torch.Tensor,
     _lib.call("pylon_sample", out.data_ptr(), logits.data_ptr(), rows, vocab, logits.stride(0),
               _dev(temperature, "temperature", torch.float32), _dev(top_p, "top_p", torch.float32),
               _dev(uniform, "uniform", torch.float32), chosen_ptr, place_ptr, _stream())
+    return out
+
+
+def qkv_prepare_wide(qkv: torch.Tensor, q_out: torch.Tensor, k_cache: Optional[torch.Tensor],
+                     v_cache: Optional[torch.Tensor], *, n_heads: int, n_kv_heads: int, head_dim: int, v_dim: int,
+                     q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor], eps: float,
+                     inv_freq: Optional[torch.Tensor], rot_dim: int, interleaved: bool,
+                     positions: Optional[torch.Tensor], slot_map: Optional[torch.Tensor], store_kv: bool) -> None:
+    """q/k/v preparation with norms over whole projections: ``q_weight`` (float32, all heads of q
+    side by side) and ``k_weight`` norm the whole q row and the whole k row of a token (None: no
+    norm); the first ``rot_dim`` elements of every head of q and k are rotated by ``position *
+    inv_freq[i]``, pairing neighbours (``interleaved``) or halves; q goes to ``q_out``, k and v
+    (heads of ``v_dim`` elements) into the tokens' cache slots."""
+    if qkv.dim() != 2 or qkv.stride(1) != 1:
+        raise KernelError("qkv_prepare_wide takes a 2-D projection output with contiguous rows")
+    tokens, width = qkv.shape
+    q_size, k_size, v_size = n_heads * head_dim, n_kv_heads * head_dim, n_kv_heads * v_dim
+    if width != q_size + (k_size + v_size if store_kv else 0):
+        raise KernelError(f"qkv_prepare_wide: projection width {width} does not match the heads")
+    if q_out.shape != (tokens, n_heads, head_dim) or q_out.dtype != qkv.dtype:
+        raise KernelError("qkv_prepare_wide: q_out has the wrong shape or dtype")
+    if q_weight is not None and q_weight.shape != (q_size,):
+        raise KernelError(f"qkv_prepare_wide: q_weight must have shape ({q_size},)")
+    if k_weight is not None and k_weight.shape != (k_size,):
+        raise KernelError(f"qkv_prepare_wide: k_weight must have shape ({k_size},)")
+    if rot_dim and (inv_freq is None or inv_freq.numel() != rot_dim // 2 or positions is None
+                    or positions.numel() != tokens):
+        raise KernelError("qkv_prepare_wide: a rotation needs rot_dim/2 frequencies and one position per token")
+    if store_kv:
+        if k_cache is None or v_cache is None or slot_map is None or slot_map.numel() != tokens:
+            raise KernelError("qkv_prepare_wide: storing needs k_cache, v_cache and one slot per token")
+        if k_cache.dtype != qkv.dtype or k_cache.shape[-2:] != (n_kv_heads, head_dim):
+            raise KernelError(f"qkv_prepare_wide: k_cache must be [..., {n_kv_heads}, {head_dim}] of {qkv.dtype}")
+        if v_cache.dtype != qkv.dtype or v_cache.shape[-2:] != (n_kv_heads, v_dim):
+            raise KernelError(f"qkv_prepare_wide: v_cache must be [..., {n_kv_heads}, {v_dim}] of {qkv.dtype}")
+    if not qkv.is_cuda:
+        raise KernelError("qkv must live on the GPU; there is no CPU path")
+    _lib.call("pylon_qkv_prepare_wide", _dev(q_out, "q_out"), _dev(k_cache if store_kv else None, "k_cache"),
+              _dev(v_cache if store_kv else None, "v_cache"), qkv.data_ptr(), dtype_code(qkv.dtype), qkv.stride(0),
+              _dev(q_weight, "q_weight", torch.float32), _dev(k_weight, "k_weight", torch.float32), float(eps),
+              _dev(inv_freq, "inv_freq", torch.float32), int(rot_dim), 1 if interleaved else 0,
+              _dev(positions, "positions", torch.int32), _dev(slot_map if store_kv else None, "slot_map", torch.int32),
+              tokens, n_heads, n_kv_heads, head_dim, v_dim, 1 if store_kv else 0, _stream())
+
+
+def latent_prepare(down: torch.Tensor, cache: Optional[torch.Tensor], slot_map: Optional[torch.Tensor], *,
+                   q_rank: int, kv_rank: int, n_gate: int, q_weight: torch.Tensor, c_weight: torch.Tensor,
+                   eps: float, out_dtype: torch.dtype):
+    """From the float32 sums ``down`` ``[tokens, q_rank + kv_rank + n_gate]`` of a fused down
+    projection: the normed query latent ``[tokens, q_rank]`` in ``out_dtype``, the normed key/value
+    latent into ``cache`` (``[..., kv_rank]`` of ``out_dtype``) at the tokens' slots (``cache``
+    None: nothing is stored), and ``sigmoid`` of the last ``n_gate`` numbers as float32
+    ``[tokens, n_gate]`` (None without gates).  Both norms in float32."""
+    if down.dim() != 2 or down.dtype != torch.float32 or down.stride(1) != 1:
+        raise KernelError("latent_prepare takes float32 sums [tokens, width] with contiguous rows")
+    tokens, width = down.shape
+    if width != q_rank + kv_rank + n_gate:
+        raise KernelError(f"latent_prepare: rows of {width} numbers, expected {q_rank + kv_rank + n_gate}")
+    if q_weight.shape != (q_rank,) or c_weight.shape != (kv_rank,):
+        raise KernelError("latent_prepare: the norms' weights have the latents' sizes")
+    store = cache is not None
+    if store and (slot_map is None or slot_map.numel() != tokens or cache.dtype != out_dtype
+                  or cache.shape[-1] != kv_rank or not cache.is_contiguous()):
+        raise KernelError("latent_prepare: the cache must be [..., kv_rank] of the output type, with one slot per token")
+    q_latent = torch.empty((tokens, q_rank), dtype=out_dtype, device=down.device)
+    gate = torch.empty((tokens, n_gate), dtype=torch.float32, device=down.device) if n_gate else None
+    _lib.call("pylon_latent_prepare", _dev(q_latent, "q_latent"), _dev(cache, "cache"), _dev(gate, "gate"),
+              _dev(down, "down") if down.is_contiguous() else down.data_ptr(), down.stride(0), dtype_code(out_dtype),
+              _dev(q_weight, "q_weight", torch.float32), _dev(c_weight, "c_weight", torch.float32), float(eps),
+              _dev(slot_map if store else None, "slot_map", torch.int32), tokens, q_rank, kv_rank, n_gate,
+              1 if store else 0, _stream())
+    return q_latent, gate
+
+
+HEAD_PROJECT_ROWS = 64  # up to this many tokens the per-head products of bfloat16 run on the engine's own kernel
+
+
+def head_project(x: torch.Tensor, m: torch.Tensor, *, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``out[t, h] = gate[t, h] * x[t, h] @ m[h]`` for ``x`` ``[tokens, heads, n_in]`` (the heads of
+    a row side by side, rows maybe apart) and ``m`` ``[heads, n_in, n_out]``; ``gate`` float32
+    ``[tokens, heads]`` or None.  float32 operands and up to 64 bfloat16 tokens: the engine's
+    kernel (float sums in the order of ``n_in``, one rounding); more bfloat16 tokens: the
+    library's batched product, then the gate."""
+    if x.dim() != 3 or m.dim() != 3 or m.shape[0] != x.shape[1] or m.shape[1] != x.shape[2]:
+        raise KernelError(f"head_project: cannot multiply {tuple(x.shape)} head by head by {tuple(m.shape)}")
+    tokens, heads, n_in = x.shape
+    n_out = m.shape[2]
+    if x.stride(2) != 1 or x.stride(1) != n_in or not m.is_contiguous() or not x.is_cuda:
+        raise KernelError("head_project: the heads of a row lie side by side, m is contiguous, both on the GPU")
+    if gate is not None and (gate.shape != (tokens, heads) or gate.dtype != torch.float32):
+        raise KernelError("head_project: gate must be float32 [tokens, heads]")
+    if x.dtype == torch.bfloat16 and m.dtype == torch.bfloat16 and tokens > HEAD_PROJECT_ROWS:
+        out = torch.empty((tokens, heads, n_out), dtype=x.dtype, device=x.device)
+        torch.bmm(x.transpose(0, 1), m, out=out.transpose(0, 1))
+        if gate is not None:
+            _lib.call("pylon_gate_heads", _dev(out, "out"), dtype_code(out.dtype), _dev(gate, "gate", torch.float32),
+                      tokens * heads, n_out, _stream())
+        return out
+    out = torch.empty((tokens, heads, n_out), dtype=x.dtype, device=x.device)
+    _lib.call("pylon_head_project", _dev(out, "out"), x.data_ptr(), dtype_code(x.dtype),
+              x.stride(0) if tokens > 1 else heads * n_in, _dev(m, "m"), dtype_code(m.dtype),
+              _dev(gate, "gate", torch.float32), tokens, heads, n_in, n_out, _stream())
+    return out
+
+
+def route_top(logits: torch.Tensor, bias: Optional[torch.Tensor], *, n_experts: int, top: int,
+              shared_gate: bool):
+    """From float32 router logits ``[tokens, n_experts (+ 1 with shared_gate)]``: the ``top``
+    experts with the largest ``logit + bias`` per token (int32 ``[tokens, top]``, the lower index
+    among equals), the softmax over those alone (float32 ``[tokens, top]``), and ``sigmoid`` of the
+    last column (float32 ``[tokens]``, or None)."""
+    if logits.dim() != 2 or logits.dtype != torch.float32 or logits.stride(1) != 1:
+        raise KernelError("route_top takes float32 logits [tokens, experts]")
+    tokens = logits.shape[0]
+    if logits.shape[1] != n_experts + (1 if shared_gate else 0):
+        raise KernelError("route_top: the logits' columns do not match the experts")
+    if bias is not None and bias.shape != (n_experts,):
+        raise KernelError("route_top: one bias per expert")
+    experts = torch.empty((tokens, top), dtype=torch.int32, device=logits.device)
+    weights = torch.empty((tokens, top), dtype=torch.float32, device=logits.device)
+    gate = torch.empty((tokens,), dtype=torch.float32, device=logits.device) if shared_gate else None
+    _lib.call("pylon_route_top", _dev(experts, "experts"), _dev(weights, "weights"), _dev(gate, "gate"),
+              logits.data_ptr(), logits.stride(0), _dev(bias, "bias", torch.float32), tokens, n_experts, top,
+              _stream())
+    return experts, weights, gate
+
+
+def expert_gate_up(x: torch.Tensor, gate_up: torch.Tensor, experts: torch.Tensor, *, n_experts: int,
+                   ff: int) -> torch.Tensor:
+    """``silu(W_gate[e] x_t) * (W_up[e] x_t)`` for every token and each of its chosen experts:
+    ``gate_up`` is ``[n_experts * 2 ff, width]`` (an expert's gate rows, then its up rows);
+    returns ``[tokens * top, ff]`` of ``x``'s type, float sums rounded once."""
+    tokens, width = x.shape
+    top = experts.shape[1]
+    if gate_up.shape != (n_experts * 2 * ff, width) or gate_up.stride(1) != 1 or x.stride(1) != 1:
+        raise KernelError("expert_gate_up: the experts' matrix must be [experts * 2 ff, width]")
+    if experts.shape[0] != tokens or experts.dtype != torch.int32 or not experts.is_contiguous():
+        raise KernelError("expert_gate_up: experts must be int32 [tokens, top]")
+    hidden = torch.empty((tokens * top, ff), dtype=x.dtype, device=x.device)
+    _lib.call("pylon_expert_gate_up", _dev(hidden, "hidden"), x.data_ptr(), dtype_code(x.dtype), x.stride(0),
+              gate_up.data_ptr(), dtype_code(gate_up.dtype), gate_up.stride(0), _dev(experts, "experts"), tokens, top,
+              ff, width, _stream())
+    return hidden
+
+
+def expert_down(hidden: torch.Tensor, down: torch.Tensor, experts: torch.Tensor, weights: torch.Tensor, *,
+                n_experts: int, width: int, shared: Optional[torch.Tensor] = None,
+                shared_gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """float32 ``[tokens, width]``: ``sum_s weights[t, s] W_down[e_s] hidden[(t, s)]`` with ``down``
+    ``[n_experts * width, ff]``, plus ``shared_gate[t] * shared[t]`` (``shared`` float32
+    ``[tokens, width]``; without the gate it is added as it is)."""
+    tokens, top = experts.shape
+    ff = hidden.shape[1]
+    if hidden.shape[0] != tokens * top or not hidden.is_contiguous():
+        raise KernelError("expert_down: hidden must be [tokens * top, ff]")
+    if down.shape != (n_experts * width, ff) or down.stride(1) != 1:
+        raise KernelError("expert_down: the experts' matrix must be [experts * width, ff]")
+    if weights.shape != (tokens, top) or weights.dtype != torch.float32:
+        raise KernelError("expert_down: weights must be float32 [tokens, top]")
+    if shared is not None and (shared.shape != (tokens, width) or shared.dtype != torch.float32):
+        raise KernelError("expert_down: the shared expert's output must be float32 [tokens, width]")
+    if shared_gate is not None and (shared is None or shared_gate.numel() != tokens):
+        raise KernelError("expert_down: one gate per token, and only with a shared output")
+    out = torch.empty((tokens, width), dtype=torch.float32, device=hidden.device)
+    _lib.call("pylon_expert_down", _dev(out, "out"), _dev(hidden, "hidden"), dtype_code(hidden.dtype),
+              down.data_ptr(), dtype_code(down.dtype), down.stride(0), _dev(experts, "experts", torch.int32),
+              _dev(weights, "weights", torch.float32), _dev(shared, "shared", torch.float32),
+              _dev(shared_gate, "shared_gate", torch.float32), tokens, top, ff, width, _stream())
     return out
 
 

@@ -1,5 +1,5 @@
 """The parts layers are assembled from; importing this package registers the built-in ones."""
-from . import attention, block, feed_forward, logits, norm, position, retention, short_conv  # noqa: F401
+from . import attention, block, feed_forward, latent_attention, logits, mixture, norm, position, retention, short_conv  # noqa: F401
 from .base import KVRequirement, Normed, Part, StateRequirement, requirement_list, summed
 from .registry import build_part, register_part, registered, unregister_part
 

@@ -6,6 +6,12 @@
 position encoding of q and k, k and v stored at the tokens' cache slots, causal softmax
 attention of every token over its request's keys, output projection.  A run that borrows
 another run's cache projects q only and stores nothing.
+
+The spec may ask instead for one norm over the whole q projection and one over the whole k
+projection (``qk_norm_over="projection"``), for a rotation that pairs neighbouring elements (the
+position part's ``interleaved``) over a part of the head, for values of another size than keys,
+and for keys visible inside the query's chunk of positions only (``chunk``); these go through
+:func:`ops.qkv_prepare_wide` and the same attention kernels, which take the mask as one integer.
 """
 from __future__ import annotations
 
@@ -31,27 +37,42 @@ class Attention(Part):
             )
         if spec.window is not None and spec.window < 1:
             raise ValueError("window must be positive (or None for full attention)")
+        if spec.chunk is not None and (spec.chunk < 1 or spec.window is not None):
+            raise ValueError("chunk must be positive, and a layer has a window or chunks, not both")
+        if spec.qk_norm_over not in ("head", "projection"):
+            raise ValueError(f"qk_norm_over must be 'head' or 'projection', got {spec.qk_norm_over!r}")
+        if spec.value_dim < 1 or spec.value_dim > 512:
+            raise ValueError(f"value heads of {spec.value_dim} elements are not supported: 1 to 512")
         self.spec = spec
         self.dtype = dtype
         q, kv = spec.q_size, spec.kv_size
-        self.add_param("qkv", (q + 2 * kv, spec.hidden_size), dtype, device)
-        self.add_param("out", (spec.hidden_size, q), dtype, device)
+        self.add_param("qkv", (q + kv + spec.v_size, spec.hidden_size), dtype, device)
+        self.add_param("out", (spec.hidden_size, spec.n_heads * spec.value_dim), dtype, device)
         if spec.qk_norm:
-            self.add_param("q_norm", (spec.head_dim,), torch.float32, device, role="vector")
-            self.add_param("k_norm", (spec.head_dim,), torch.float32, device, role="vector")
+            over_heads = spec.qk_norm_over == "head"
+            self.add_param("q_norm", (spec.head_dim if over_heads else q,), torch.float32, device, role="vector")
+            self.add_param("k_norm", (spec.head_dim if over_heads else kv,), torch.float32, device, role="vector")
         self.position = self.add_child("position", build_part("position", spec.position, dtype=dtype, device=device))
+        # what the per-head preparation kernels (and the decode kernel that prepares its own
+        # operands) cover: norms head by head, halves rotated together, values as large as keys
+        self.plain = ((not spec.qk_norm or spec.qk_norm_over == "head") and spec.value_dim == spec.head_dim
+                      and not getattr(self.position, "interleaved", False))
 
     def cache_requirement(self) -> KVRequirement:
-        return KVRequirement(self.spec.n_kv_heads, self.spec.head_dim, self.spec.window)
+        spec = self.spec
+        return KVRequirement(spec.n_kv_heads, spec.head_dim, spec.window,
+                             v_head_dim=None if spec.value_dim == spec.head_dim else spec.value_dim, chunk=spec.chunk)
 
     def _span(self, ctx) -> int:
         """The most keys a token of this step attends to."""
-        return ctx.max_len if self.spec.window is None else min(ctx.max_len, self.spec.window)
+        span = self.spec.window if self.spec.window is not None else self.spec.chunk
+        return ctx.max_len if span is None else min(ctx.max_len, span)
 
     def decode_signature(self, rows: int, bound: int) -> tuple:
         """Of a bound on the lengths, a decode-only step's launches take only how the keys of
         a request are shared between workgroups and waves."""
-        span = bound if self.spec.window is None else min(bound, self.spec.window)
+        limit = self.spec.window if self.spec.window is not None else self.spec.chunk
+        span = bound if limit is None else min(bound, limit)
         return ("attention",) + tuple(ops.decode_launch(rows, self.spec.n_kv_heads, span))
 
     def forward(self, h: torch.Tensor, ctx, cache, stores: bool) -> torch.Tensor:
@@ -61,7 +82,8 @@ class Attention(Part):
         if not stores:
             weight = weight[: spec.q_size]
         rotary = self.position.rotary()
-        if ctx.decode_only and cache.k is not None and ops.decode_fused_ok(
+        mask = dict(window=spec.window, chunk=spec.chunk)
+        if self.plain and spec.chunk is None and ctx.decode_only and cache.k is not None and ops.decode_fused_ok(
                 self.dtype, cache.k, tokens=tokens, n_heads=spec.n_heads, head_dim=spec.head_dim,
                 rot_dim=rotary[1] if rotary else 0):
             # one launch adds the projection's partial sums if it comes as such, norms and
@@ -79,22 +101,34 @@ class Attention(Part):
                                            out_dtype=self.dtype)
         qkv = ops.linear(h, weight, out_dtype=self.dtype)
         q = torch.empty((tokens, spec.n_heads, spec.head_dim), dtype=self.dtype, device=h.device)
-        ops.qkv_prepare(
-            qkv, q, cache.k, cache.v,
-            n_heads=spec.n_heads, n_kv_heads=spec.n_kv_heads, head_dim=spec.head_dim,
-            q_weight=self.params.get("q_norm"), k_weight=self.params.get("k_norm"),
-            eps=spec.qk_norm_eps,
-            inv_freq=rotary[0] if rotary else None, rot_dim=rotary[1] if rotary else 0,
-            positions=ctx.positions, slot_map=cache.slot_map, store_kv=stores,
-        )
-        if ctx.decode_only and ops.decode_attention_ok(q, cache.k):
+        if self.plain:
+            ops.qkv_prepare(
+                qkv, q, cache.k, cache.v,
+                n_heads=spec.n_heads, n_kv_heads=spec.n_kv_heads, head_dim=spec.head_dim,
+                q_weight=self.params.get("q_norm"), k_weight=self.params.get("k_norm"),
+                eps=spec.qk_norm_eps,
+                inv_freq=rotary[0] if rotary else None, rot_dim=rotary[1] if rotary else 0,
+                positions=ctx.positions, slot_map=cache.slot_map, store_kv=stores,
+            )
+        else:
+            # norms over whole projections, neighbours rotated together, values of another size
+            ops.qkv_prepare_wide(
+                qkv, q, cache.k, cache.v,
+                n_heads=spec.n_heads, n_kv_heads=spec.n_kv_heads, head_dim=spec.head_dim, v_dim=spec.value_dim,
+                q_weight=self.params.get("q_norm"), k_weight=self.params.get("k_norm"), eps=spec.qk_norm_eps,
+                inv_freq=rotary[0] if rotary else None, rot_dim=rotary[1] if rotary else 0,
+                interleaved=getattr(self.position, "interleaved", False),
+                positions=ctx.positions, slot_map=cache.slot_map, store_kv=stores,
+            )
+        same_size = spec.value_dim == spec.head_dim  # the matrix-core kernels take values as large as keys
+        if same_size and ctx.decode_only and ops.decode_attention_ok(q, cache.k):
             cuts, splits = ops.decode_launch(tokens, spec.n_kv_heads, self._span(ctx))
             # in a decode-only step token t is row t
             context = ops.attention_decode(
                 q, cache.k, cache.v, cache.block_table, None, ctx.positions,
-                page_size=cache.page_size, window=spec.window, scale=spec.scale, n_splits=splits, n_cuts=cuts,
+                page_size=cache.page_size, scale=spec.scale, n_splits=splits, n_cuts=cuts, **mask,
             )
-        elif ops.prefill_attention_ok(q, cache.k, cache.block_table):
+        elif same_size and ops.prefill_attention_ok(q, cache.k, cache.block_table):
             group = spec.n_heads // spec.n_kv_heads
             rows = ops.prefill_rows(tokens, spec.n_heads, group)
             context = torch.empty_like(q)
@@ -105,26 +139,26 @@ class Attention(Part):
                 singles = 0
             if singles:
                 span = int(ctx.starts[:singles].max()) + 1
-                if spec.window is not None:
-                    span = min(span, spec.window)
+                if spec.window is not None or spec.chunk is not None:
+                    span = min(span, spec.window if spec.window is not None else spec.chunk)
                 cuts, splits = ops.decode_launch(singles, spec.n_kv_heads, span)
                 ops.attention_decode(
                     q[:singles], cache.k, cache.v, cache.block_table, None, ctx.positions[:singles],
-                    page_size=cache.page_size, window=spec.window, scale=spec.scale, n_splits=splits,
-                    n_cuts=cuts, out=context[:singles],
+                    page_size=cache.page_size, scale=spec.scale, n_splits=splits,
+                    n_cuts=cuts, out=context[:singles], **mask,
                 )
             if singles < ctx.rows:
                 tiles = ctx.token_tiles(rows // group, skip_rows=singles, fold=ops.prefill_fold(spec.n_kv_heads))
                 ops.attention_prefill(
                     q, cache.k, cache.v, cache.block_table, tiles,
-                    page_size=cache.page_size, window=spec.window, scale=spec.scale, rows=rows, out=context,
+                    page_size=cache.page_size, scale=spec.scale, rows=rows, out=context, **mask,
                 )
         else:
             context = ops.paged_attention(
                 q, cache.k, cache.v, cache.block_table, ctx.tok_row, ctx.positions,
-                page_size=cache.page_size, window=spec.window, scale=spec.scale,
+                page_size=cache.page_size, scale=spec.scale, **mask,
             )
-        return ops.linear_for_residual(context.view(tokens, spec.q_size), self.params["out"],
+        return ops.linear_for_residual(context.view(tokens, spec.n_heads * spec.value_dim), self.params["out"],
                                        out_dtype=self.dtype)
 
 

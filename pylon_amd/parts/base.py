@@ -49,10 +49,37 @@ class KVRequirement:
     head_dim: int
     window: Optional[int] = None  # keep only the last `window` tokens' entries
     v_head_dim: Optional[int] = None  # size of a value head where it differs from a key head's
+    # keep only the entries of the chunk of `chunk` positions that the next token falls into
+    # (chunks counted from the request's first token)
+    chunk: Optional[int] = None
+    # False: one entry per token only (a latent from which keys and values are both made);
+    # no tensor of values is kept, and the run's view has ``v`` None
+    values: bool = True
 
     @property
     def value_dim(self) -> int:
+        if not self.values:
+            return 0
         return self.head_dim if self.v_head_dim is None else self.v_head_dim
+
+    @property
+    def bounded(self) -> bool:
+        """Whether a request needs only a bounded number of this cache's entries."""
+        return self.window is not None or self.chunk is not None
+
+    @property
+    def span(self) -> Optional[int]:
+        """The most entries a token ever looks back over, itself included (None: all)."""
+        return self.window if self.window is not None else self.chunk
+
+    def first_needed(self, length: int) -> int:
+        """The first position that the token at position ``length`` (the next one of a request
+        that holds ``length``) still sees."""
+        if self.window is not None:
+            return max(0, length - self.window + 1)
+        if self.chunk is not None:
+            return length // self.chunk * self.chunk
+        return 0
 
 
 @dataclass(frozen=True)

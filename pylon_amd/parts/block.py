@@ -23,12 +23,16 @@ class PreNormBlock(Part):
         kw = dict(dtype=dtype, device=device)
         self.mixer_norm = self.add_child("mixer_norm", build_part("norm", spec.mixer_norm, **kw))
         self.mixer = self.add_child("mixer", build_part("mixer", spec.mixer, **kw))
-        self.feed_forward_norm = self.add_child(
-            "feed_forward_norm", build_part("norm", spec.feed_forward_norm, **kw)
-        )
-        self.feed_forward = self.add_child(
-            "feed_forward", build_part("feed_forward", spec.feed_forward, **kw)
-        )
+        if (spec.feed_forward is None) != (spec.feed_forward_norm is None):
+            raise ValueError("a feed-forward and its norm come together or not at all")
+        self.feed_forward = None  # a layer may consist of its mixer alone
+        if spec.feed_forward is not None:
+            self.feed_forward_norm = self.add_child(
+                "feed_forward_norm", build_part("norm", spec.feed_forward_norm, **kw)
+            )
+            self.feed_forward = self.add_child(
+                "feed_forward", build_part("feed_forward", spec.feed_forward, **kw)
+            )
 
     def cache_requirement(self):
         return self.mixer.cache_requirement()
@@ -41,6 +45,8 @@ class PreNormBlock(Part):
                 stores: bool) -> Tuple[torch.Tensor, torch.Tensor]:
         h = self.mixer_norm.add_forward(resid, delta)
         mixed = self.mixer.forward(h, ctx, cache, stores)
+        if self.feed_forward is None:
+            return resid, mixed
         h = self.feed_forward_norm.add_forward(resid, mixed)
         return resid, self.feed_forward.forward(h, ctx)
 

@@ -3,7 +3,7 @@ from __future__ import annotations
 
 import torch
 
-from ..config.specs import LogitScaleSpec
+from ..config.specs import LogitScaleSpec, LogitSoftcapSpec
 from ..kernels import ops
 from .base import Part
 from .registry import register_part
@@ -22,4 +22,19 @@ class LogitScale(Part):
         return logits
 
 
+class LogitSoftcap(Part):
+    """``logits <- cap * tanh(logits / cap)``, in place."""
+
+    def __init__(self, spec: LogitSoftcapSpec, *, dtype: torch.dtype, device) -> None:
+        super().__init__()
+        if not spec.cap > 0:
+            raise ValueError(f"a soft cap must be positive, got {spec.cap!r}")
+        self.spec = spec
+
+    def forward(self, logits: torch.Tensor, ctx) -> torch.Tensor:
+        ops.softcap_(logits, self.spec.cap)
+        return logits
+
+
 register_part("logits", "scale", LogitScale, replace=True)
+register_part("logits", "softcap", LogitSoftcap, replace=True)

@@ -1,0 +1,63 @@
+"""A mixture of gated feed-forward experts with an optional shared expert.
+
+Router logits ``W_r h + b`` are a float32 product (the router's matrix is kept in float32 whatever
+the model's type; with a gated shared expert its gate vector is one more row of the same matrix);
+one kernel picks every token's ``top`` experts and the softmax over their logits; one computes
+``silu(gate) * up`` of every (token, chosen expert) from the experts' fused gate/up matrix, and one
+applies the chosen experts' down matrices, weights the results and adds the shared expert's output
+times its gate.  The shared expert itself is an ordinary gated feed-forward on the engine's
+product kernels.  The result is float32 and goes to the residual sum unrounded.  A token's
+output does not depend on which other tokens share its step: every kernel here works token by
+token with a fixed order of additions.
+"""
+from __future__ import annotations
+
+import torch
+
+from ..config.specs import MixtureFeedForwardSpec
+from ..kernels import ops, plan
+from .base import Part
+from .registry import register_part
+
+
+class MixtureFeedForward(Part):
+    def __init__(self, spec: MixtureFeedForwardSpec, *, dtype: torch.dtype, device) -> None:
+        super().__init__()
+        if not 1 <= spec.top <= spec.n_experts:
+            raise ValueError(f"a token uses 1 to {spec.n_experts} of {spec.n_experts} experts, not {spec.top}")
+        if spec.n_experts > 512 or spec.top > 32:
+            raise ValueError("the router kernel takes up to 512 experts and up to 32 of them a token")
+        if spec.shared_size is None and spec.shared_gate:
+            raise ValueError("a gate of the shared expert needs a shared expert")
+        self.spec = spec
+        self.dtype = dtype
+        width, ff = spec.hidden_size, spec.expert_size
+        self.router_rows = spec.n_experts + (1 if spec.shared_gate else 0)
+        self.add_param("router", (self.router_rows, width), torch.float32, device, role="vector")
+        if spec.router_bias:
+            self.add_param("router_bias", (spec.n_experts,), torch.float32, device, role="vector")
+        # expert e: rows [e * 2 ff, e * 2 ff + ff) its gate, the next ff its up; rows [e * width, ...) its down
+        self.add_param("gate_up", (spec.n_experts * 2 * ff, width), dtype, device)
+        self.add_param("down", (spec.n_experts * width, ff), dtype, device)
+        if spec.shared_size is not None:
+            element_size = torch.empty((), dtype=dtype).element_size()
+            self.add_param("shared_gate_up", (2 * spec.shared_size, width), dtype, device,
+                           row_padding=plan.gated_row_padding(width, element_size))
+            self.add_param("shared_down", (width, spec.shared_size), dtype, device)
+
+    def forward(self, h: torch.Tensor, ctx) -> torch.Tensor:
+        spec = self.spec
+        logits = ops.gemm_tiled(h, self.params["router"], out_dtype=torch.float32)
+        experts, weights, shared_gate = ops.route_top(
+            logits, self.params.get("router_bias"), n_experts=spec.n_experts, top=spec.top,
+            shared_gate=spec.shared_gate)
+        hidden = ops.expert_gate_up(h, self.params["gate_up"], experts, n_experts=spec.n_experts, ff=spec.expert_size)
+        shared = None
+        if spec.shared_size is not None:
+            shared_hidden = ops.linear_glu(h, self.params["shared_gate_up"], out_dtype=self.dtype)
+            shared = ops.linear(shared_hidden, self.params["shared_down"], out_dtype=torch.float32)
+        return ops.expert_down(hidden, self.params["down"], experts, weights, n_experts=spec.n_experts,
+                               width=spec.hidden_size, shared=shared, shared_gate=shared_gate)
+
+
+register_part("feed_forward", "mixture", MixtureFeedForward, replace=True)

@@ -1,6 +1,7 @@
 """RMSNorm over the hidden axis (/root/reference/src/pylon/model/layers.py:30-40):
 ``y = x / sqrt(mean(x^2) + eps) * w`` in float32, rounded once to the activation dtype.
-The weight is kept in float32 whatever the model's dtype, as the reference keeps it."""
+The weight is kept in float32 whatever the model's dtype, as the reference keeps it.  With
+``weight_offset`` the stored weight is a distance from that number: ``y = ... * (offset + w)``."""
 from __future__ import annotations
 
 from typing import Optional
@@ -19,16 +20,28 @@ class RMSNorm(Part):
         self.spec = spec
         self.dtype = dtype
         self.add_param("weight", (spec.dim,), torch.float32, device, role="vector")
+        self._shifted = None  # (version of the parameter, weight + offset)
+
+    def weight(self) -> torch.Tensor:
+        """What multiplies: the stored weight, plus ``weight_offset`` for a norm whose weights are
+        stored as their distance from it (formed in float32, anew when the parameter is written)."""
+        stored = self.params["weight"]
+        if not self.spec.weight_offset:
+            return stored
+        key = (stored.data_ptr(), stored._version)
+        if self._shifted is None or self._shifted[0] != key:
+            self._shifted = (key, stored + self.spec.weight_offset)
+        return self._shifted[1]
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        return ops.rmsnorm(x, self.params["weight"], self.spec.eps, out_dtype=self.dtype)
+        return ops.rmsnorm(x, self.weight(), self.spec.eps, out_dtype=self.dtype)
 
     def add_forward(self, resid: torch.Tensor, delta, *,
                     row_idx: Optional[torch.Tensor] = None) -> torch.Tensor:
         if isinstance(delta, Normed):
-            return ops.add_normed_rmsnorm(resid, delta.value, self.params["weight"], self.spec.eps, self.dtype,
+            return ops.add_normed_rmsnorm(resid, delta.value, self.weight(), self.spec.eps, self.dtype,
                                           post_gain=delta.gain, post_eps=delta.eps, row_idx=row_idx)
-        return ops.add_rmsnorm(resid, delta, self.params["weight"], self.spec.eps, self.dtype,
+        return ops.add_rmsnorm(resid, delta, self.weight(), self.spec.eps, self.dtype,
                                row_idx=row_idx)
 
 

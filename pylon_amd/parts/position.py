@@ -5,6 +5,8 @@
 (float32), and element ``i`` of a head is rotated together with element ``i + d/2``.
 The reference gathers cos/sin from tables of ``max_position_embeddings`` rows; here the
 fused q/k kernel forms the angle from the position, which gives the same float32 value.
+With ``interleaved`` element ``2i`` is rotated together with its neighbour ``2i + 1`` instead
+(the part's ``interleaved`` attribute says so to the mixer, which picks a kernel that does it).
 """
 from __future__ import annotations
 
@@ -23,8 +25,15 @@ class RotaryPosition(Part):
         if spec.rotary_dim < 2 or spec.rotary_dim % 2:
             raise ValueError("rotary_dim must be even and at least 2")
         self.spec = spec
-        exponents = torch.arange(0, spec.rotary_dim, 2, dtype=torch.float32) / spec.rotary_dim
-        inv_freq = 1.0 / (torch.tensor(spec.theta, dtype=torch.float32) ** exponents)
+        self.interleaved = spec.interleaved
+        if spec.interleaved:
+            # neighbours (2i, 2i + 1) turn together; frequencies theta ** (-2i/d) formed in double
+            # precision and rounded to float32 once
+            exponents = torch.arange(0, spec.rotary_dim, 2, dtype=torch.float64) / spec.rotary_dim
+            inv_freq = (torch.tensor(spec.theta, dtype=torch.float64) ** -exponents).to(torch.float32)
+        else:
+            exponents = torch.arange(0, spec.rotary_dim, 2, dtype=torch.float32) / spec.rotary_dim
+            inv_freq = 1.0 / (torch.tensor(spec.theta, dtype=torch.float32) ** exponents)
         self.inv_freq = inv_freq.to(device)
 
     def rotary(self) -> Optional[Tuple[torch.Tensor, int]]:
@@ -35,6 +44,7 @@ class NoPosition(Part):
     def __init__(self, spec: PositionSpec, *, dtype: torch.dtype, device) -> None:
         super().__init__()
         self.spec = spec
+        self.interleaved = False
 
     def rotary(self):
         return None

@@ -33,7 +33,8 @@ def draw_tensor(seed: int, name: str, target, sigma: float, norm_jitter: float, 
                 draw_on=None) -> None:
     """The one rule of the random-weights mode: fill ``out`` (of the target's shape, on any
     device, of any float type) with tensor ``name`` of seed ``seed``.  ``normal``:
-    N(0, sigma^2); ``ones`` / ``ones_jitter``: 1, or 1 + norm_jitter * N(0, 1).  The numbers
+    N(0, sigma^2); ``ones`` / ``ones_jitter``: 1, or 1 + norm_jitter * N(0, 1); ``zeros_jitter``: 0, or
+    norm_jitter * N(0, 1).  The numbers
     come from a generator keyed by (seed, name) on the device ``draw_on`` (default: where
     ``out`` lives): drawn on the CPU they are the numbers of the folder that
     :func:`write_random_model` writes; drawn on a GPU they follow the same rule with other
@@ -43,11 +44,15 @@ def draw_tensor(seed: int, name: str, target, sigma: float, norm_jitter: float, 
     if target.init in ("ones", "ones_jitter") and not (target.init == "ones_jitter" and norm_jitter):
         out.fill_(1.0)
         return
-    if target.init not in ("normal", "ones_jitter"):
+    if target.init == "zeros_jitter" and not norm_jitter:  # a norm weight stored as its distance from one
+        out.fill_(0.0)
+        return
+    if target.init not in ("normal", "ones_jitter", "zeros_jitter"):
         raise ValueError(f"unknown init rule {target.init!r} for {name}")
     where = torch.device(draw_on) if draw_on is not None else out.device
     gen = _generator(seed, name, where)
-    scale, shift = (sigma, 0.0) if target.init == "normal" else (norm_jitter, 1.0)
+    scale, shift = {"normal": (sigma, 0.0), "ones_jitter": (norm_jitter, 1.0), "zeros_jitter": (norm_jitter, 0.0)}[
+        target.init]
     if out.is_contiguous():
         flat = out.view(-1)
         for start in range(0, flat.numel(), _SLAB):
