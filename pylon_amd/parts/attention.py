@@ -30,11 +30,15 @@ class Attention(Part):
         super().__init__()
         if spec.n_heads % spec.n_kv_heads:
             raise ValueError("The number of Q heads must be divisible by the number of KV heads.")
-        if spec.head_dim % 16 or not 16 <= spec.head_dim <= 512:
+        per_head = (not spec.qk_norm or spec.qk_norm_over == "head") and not getattr(spec.position, "interleaved", False) \
+            and spec.value_dim == spec.head_dim
+        if per_head and (spec.head_dim % 16 or not 16 <= spec.head_dim <= 512):
             raise ValueError(
                 f"head_dim {spec.head_dim} is not supported: the attention kernels take "
                 "multiples of 16 from 16 to 512"
             )
+        if not 1 <= spec.head_dim <= 512:
+            raise ValueError(f"head_dim {spec.head_dim} is not supported: 1 to 512")
         if spec.window is not None and spec.window < 1:
             raise ValueError("window must be positive (or None for full attention)")
         if spec.chunk is not None and (spec.chunk < 1 or spec.window is not None):

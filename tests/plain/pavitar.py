@@ -104,17 +104,22 @@ def gated_expert(h, w, prefix):
     return (silu(h @ w[prefix + "gate"].T) * (h @ w[prefix + "up"].T)) @ w[prefix + "down"].T
 
 
-def route(h, w, prefix, top):
-    """(experts [tokens, top], weights [tokens, top]): the largest logits, softmax over them."""
+def route(h, w, prefix, top, margins=None):
+    """(experts [tokens, top], weights [tokens, top]): the largest logits, softmax over them.
+    ``margins`` (a list) receives, per token, by how much the last chosen logit leads the first
+    that is left out (infinite when every expert is chosen)."""
     z = h @ w[prefix + "router"].T + w[prefix + "router.b"]
+    if margins is not None:
+        ranked = -np.sort(-z, axis=-1)
+        margins.append(ranked[:, top - 1] - ranked[:, top] if top < z.shape[1] else np.full(len(z), np.inf))
     order = np.argsort(-z, axis=-1, kind="stable")[:, :top]
     chosen = np.take_along_axis(z, order, axis=-1)
     e = np.exp(chosen - chosen.max(axis=-1, keepdims=True))
     return order, e / e.sum(axis=-1, keepdims=True)
 
 
-def mixture(h, w, prefix, mlp):
-    experts, weights = route(h, w, prefix, mlp["router"]["top"])
+def mixture(h, w, prefix, mlp, margins=None):
+    experts, weights = route(h, w, prefix, mlp["router"]["top"], margins)
     out = np.zeros((h.shape[0], w[prefix + "e0.down"].shape[0]))
     for t in range(h.shape[0]):
         for e, p in zip(experts[t], weights[t]):
@@ -137,8 +142,9 @@ def layer_runs(config):
     return runs + [(i, False) for i in range(stop, count)]
 
 
-def forward(config, w, tokens, *, keep_layers: bool = False):
-    """Logits [tokens, vocab] of one whole sequence (and the stream after every layer run)."""
+def forward(config, w, tokens, *, keep_layers: bool = False, margins=None):
+    """Logits [tokens, vocab] of one whole sequence (and the stream after every layer run).
+    ``margins`` (a list) receives every router's margins, see :func:`route`."""
     eps = config["norm"]["eps"]
     x = w["embed"][np.asarray(tokens)]
     embedded = x.copy()
@@ -152,9 +158,10 @@ def forward(config, w, tokens, *, keep_layers: bool = False):
         x = x + mixer(h, w, f"l{index}.mix.", layer["mixer"], eps)
         if layer.get("mlp") is not None:
             h = norm_around_zero(x, w[f"l{index}.norm2"], eps)
-            x = x + mixture(h, w, f"l{index}.mlp.", layer["mlp"])
+            x = x + mixture(h, w, f"l{index}.mlp.", layer["mlp"], margins)
         kept.append(x.copy())
     logits = norm_around_zero(x, w["final.norm"], eps) @ w["embed"].T
-    cap = config["logit_softcap"]
-    logits = cap * np.tanh(logits / cap)
+    cap = config.get("logit_softcap")
+    if cap is not None:
+        logits = cap * np.tanh(logits / cap)
     return (logits, np.stack(kept)) if keep_layers else logits
