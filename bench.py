@@ -2,7 +2,7 @@
 and uniform-random token ids, on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L]
-                    [--shape 4b|8b|32b] [--prompt-len N] [--design vupuzen [--design-shapes 8b,...]]
+                    [--shape 4b|8b|32b] [--prompt-len N] [--design vupuzen|pavitar [--design-shapes 8b,...]]
 
 Everything goes the product's own way.  Start-up is ``Runner.from_random``: the fit check,
 the measured activation headroom, the page pool sized from the card's memory and the decode
@@ -307,6 +307,31 @@ def vupuzen_json(shape: dict, layers: int) -> dict:
             "layers": [retention if i % 4 == 0 else attention for i in range(layers)]}
 
 
+def pavitar_json(shape: dict, layers: int) -> dict:
+    """A Pavitar configuration of the shape's layer sizes: every fourth layer chunked attention
+    with the shape's heads (half of every head rotated), the others latent attention with as many
+    heads over a latent of 256 numbers (the largest the matrix-core attention kernels take) and a
+    query latent of 1,024; chunks and windows of 1,024 positions; a mixture of 32 experts, 4 a
+    token, whose chosen experts and shared expert together are about as large as the shape's
+    feed-forward; the shape's vocabulary.  Of ``layers`` runs, the middle stretch runs twice over
+    the same weights (a quarter fewer layers own weights)."""
+    width, hd, heads = shape["hidden_size"], shape["head_dim"], shape["num_attention_heads"]
+    expert = max(64, shape["intermediate_size"] // 6 // 64 * 64)
+    mlp = {"kind": "moe", "expert": {"ff": expert}, "router": {"experts": 32, "top": 4}, "shared": {"ff": 2 * expert}}
+    attention = {"type": "attention", "mixer": {
+        "heads": heads, "kv_heads": shape["num_key_value_heads"], "dim": hd, "vdim": hd, "scale": hd ** -0.5,
+        "mask": {"size": 1024}, "rot": {"dims": hd // 2, "base": 1000000.0}}, "mlp": mlp}
+    latent = {"type": "latent_attention", "mixer": {
+        "heads": heads, "dim": hd, "vdim": hd, "q_rank": 1024, "kv_rank": 256, "scale": hd ** -0.5,
+        "mask": {"size": 1024}}, "mlp": mlp}
+    again = layers // 4  # this many layers run twice
+    own = layers - again
+    start = (own - again) // 2
+    return {"architecture": "Pavitar", "vocab": shape["vocab_size"], "width": width, "norm": {"eps": 1e-6},
+            "logit_softcap": 30.0, "loop": {"start": start, "stop": start + again, "times": 2 if again else 1},
+            "layers": [attention if i % 4 == 0 else latent for i in range(own)]}
+
+
 def design_steps(runner, vocab: int, batch: int, prompt_len: int, steps: int, warmup: int, seed: int) -> dict:
     """Milliseconds of one prompt step of ``prompt_len`` tokens (median of five), and of a
     decode step of ``batch`` requests behind such prompts (mean of ``steps``), through the step
@@ -348,10 +373,10 @@ def design_steps(runner, vocab: int, batch: int, prompt_len: int, steps: int, wa
 
 
 def design_main(args) -> int:
-    """``--design vupuzen``: prefill and decode of Vupuzen models of random weights at the layer
-    sizes of ``--shape`` (and of the other shapes named by ``--design-shapes``), beside the
-    Qwen3 model of the same sizes and number of layers, both through the same step function
-    over pages of 256 tokens with decode graphs."""
+    """``--design vupuzen|pavitar``: prefill and decode of models of that design of random weights
+    at the layer sizes of ``--shape`` (and of the other shapes named by ``--design-shapes``),
+    beside the Qwen3 model of the same sizes and number of layer runs, both through the same step
+    function over pages of 256 tokens with decode graphs."""
     import torch
 
     from pylon_amd.config import PylonConfig
@@ -365,7 +390,8 @@ def design_main(args) -> int:
         shape = SHAPES[name]
         layers = args.layers or 8
         pages = (args.batch + 1) * (-(-(prompt_len + steps + warmup + 8) // PAGE_SIZE) + 1)
-        for design, raw in (("vupuzen", vupuzen_json(shape, layers)), ("qwen3", config_json(shape, layers))):
+        mine_json = vupuzen_json(shape, layers) if args.design == "vupuzen" else pavitar_json(shape, layers)
+        for design, raw in ((args.design, mine_json), ("qwen3", config_json(shape, layers))):
             config = PylonConfig(dtype=args.dtype, max_batch_size=args.batch + 1, max_queue_size=args.batch + 1,
                                  page_size=PAGE_SIZE, prefill_chunk_size=prompt_len, num_pages=pages,
                                  cuda_graphs=not args.no_graphs)
@@ -375,17 +401,17 @@ def design_main(args) -> int:
             points[f"{design}_{name}"] = point
             del runner
             torch.cuda.empty_cache()
-        mine, theirs = points[f"vupuzen_{name}"], points[f"qwen3_{name}"]
+        mine, theirs = points[f"{args.design}_{name}"], points[f"qwen3_{name}"]
         points[f"ratio_{name}"] = {"prefill": round(mine["prefill_tokens_per_s"] / theirs["prefill_tokens_per_s"], 3),
                                    "decode": round(mine["decode_tokens_per_s"] / theirs["decode_tokens_per_s"], 3)}
         if record is None:
             record = {
-                "metric": f"decode tokens/s, Vupuzen at the Qwen3-{name.upper()} layer sizes, {layers} layers, "
+                "metric": f"decode tokens/s, {args.design.capitalize()} at the Qwen3-{name.upper()} layer sizes, {layers} layers, "
                           f"batch {args.batch}, {prompt_len}-token prompts",
                 "value": mine["decode_tokens_per_s"], "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
                 "ms_per_step": mine["decode_ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
                 "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
-                "config": {"model": f"vupuzen-{name}-sizes-random", "layers": layers, "global_batch": args.batch,
+                "config": {"model": f"{args.design}-{name}-sizes-random", "layers": layers, "global_batch": args.batch,
                            "seq_len": prompt_len, "page_size": PAGE_SIZE, "hip_graphs": not args.no_graphs,
                            "parallelism": "single-gpu"},
             }
@@ -415,9 +441,9 @@ def main() -> int:
     parser.add_argument("--no-peaks", action="store_true", help="skip the probes of this device's own peaks")
     parser.add_argument("--mixed", action="store_true",
                         help="also time a step of --batch decoded tokens beside a 2,048-token prompt portion")
-    parser.add_argument("--design", choices=("qwen3", "vupuzen"), default="qwen3",
-                        help="vupuzen: that design beside Qwen3 at equal sizes instead of the default workload")
-    parser.add_argument("--design-shapes", default="", help="with --design vupuzen: further shapes, with commas")
+    parser.add_argument("--design", choices=("qwen3", "vupuzen", "pavitar"), default="qwen3",
+                        help="vupuzen, pavitar: that design beside Qwen3 at equal sizes instead of the default workload")
+    parser.add_argument("--design-shapes", default="", help="with another --design: further shapes, with commas")
     parser.add_argument("--prefill-only", action="store_true",
                         help="only the prefill measurement (for profiling); prints its part of the record")
     args = parser.parse_args()

@@ -256,3 +256,178 @@ extern "C" int pylon_expert_down(float* out, const void* hidden, int h_dtype, co
   }
   PYLON_LAUNCHED("expert_down");
 }
+
+// ---- many tokens: the experts' products on the matrix cores, expert by expert ------------------
+// The (token, choice) pairs are sorted by expert (on the device, by the caller); offsets[e] is the
+// first sorted pair of expert e.  A workgroup takes 64 sorted pairs of one expert and 128 output
+// columns: four waves of 32 columns each, all 64 rows, operands fetched in the shape the matrix
+// instruction wants them (a lane: 8 neighbouring elements of one row), the next 32 elements of
+// K in flight while the current ones are multiplied.  Which (expert, rows) a workgroup has it
+// finds from the offsets itself; the grid is the most tiles there can be, and the workgroups
+// beyond the last tile leave at once.  Every output element is one chain of additions along K,
+// whatever the batch.
+typedef __bf16 mx_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float mx_floatx4 __attribute__((ext_vector_type(4)));
+
+#define MX_TM 64
+#define MX_WAVE_COLS 32
+
+template <bool GLU, typename TO>
+__global__ void __launch_bounds__(256)
+grouped_rows_kernel(TO* __restrict__ out, long long ldo, const uint16_t* __restrict__ x, long long ldx,
+                    const int* __restrict__ row_index, const uint16_t* __restrict__ w, long long ldw,
+                    long long expert_rows, const int* __restrict__ offsets, int n_experts, int N, int K) {
+  constexpr int J = GLU ? 4 : 2;  // weight tiles of a wave: GLU: two of gate rows, then the two of their up rows
+  const int lane = threadIdx.x & (PYLON_WAVE - 1), wave = threadIdx.x / PYLON_WAVE;
+  const int r = lane & 15, g = lane >> 4;
+  // this workgroup's expert and rows
+  int tile = blockIdx.x, e = 0, row0 = 0, rows = 0;
+  for (; e < n_experts; ++e) {
+    const int begin = offsets[e], count = offsets[e + 1] - begin;
+    const int tiles = (count + MX_TM - 1) / MX_TM;
+    if (tile < tiles) {
+      row0 = begin + tile * MX_TM;
+      rows = count - tile * MX_TM < MX_TM ? count - tile * MX_TM : MX_TM;
+      break;
+    }
+    tile -= tiles;
+  }
+  if (e == n_experts) return;
+  const int n0 = blockIdx.y * (4 * MX_WAVE_COLS) + wave * MX_WAVE_COLS;
+  if (n0 >= N) return;
+
+  const uint16_t* xp[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    const int local = 16 * t + r < rows ? 16 * t + r : 0;  // rows past the tile's last repeat its first
+    const int m = row0 + local;
+    xp[t] = x + static_cast<size_t>(row_index != nullptr ? row_index[m] : m) * ldx + 8 * g;
+  }
+  const uint16_t* wp[J];
+#pragma unroll
+  for (int j = 0; j < J; ++j) {
+    int n = n0 + 16 * (j & 1) + r;
+    if (n >= N) n = N - 1;  // columns past the last repeat it; they are not stored
+    const size_t row = static_cast<size_t>(e) * expert_rows + (GLU && j >= 2 ? N : 0) + n;
+    wp[j] = w + row * ldw + 8 * g;
+  }
+  mx_floatx4 acc[J][4];
+#pragma unroll
+  for (int j = 0; j < J; ++j)
+#pragma unroll
+    for (int t = 0; t < 4; ++t) acc[j][t] = mx_floatx4{0.f, 0.f, 0.f, 0.f};
+
+  const mx_bf16x8 zero = __builtin_bit_cast(mx_bf16x8, uint4{0u, 0u, 0u, 0u});
+  auto fetch = [&](mx_bf16x8(&xa)[4], mx_bf16x8(&wa)[J], int k) {
+    const bool ok = k + 8 * g < K;  // K is a multiple of 8: a lane's 8 elements are all inside or all outside
+#pragma unroll
+    for (int t = 0; t < 4; ++t) xa[t] = ok ? *reinterpret_cast<const mx_bf16x8*>(xp[t] + k) : zero;
+#pragma unroll
+    for (int j = 0; j < J; ++j) wa[j] = ok ? *reinterpret_cast<const mx_bf16x8*>(wp[j] + k) : zero;
+  };
+  auto multiply = [&](const mx_bf16x8(&xa)[4], const mx_bf16x8(&wa)[J]) {
+#pragma unroll
+    for (int j = 0; j < J; ++j)
+#pragma unroll
+      for (int t = 0; t < 4; ++t) acc[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[j], xa[t], acc[j][t], 0, 0, 0);
+  };
+  mx_bf16x8 xa[4], wa[J], xb[4], wb[J];
+  fetch(xa, wa, 0);
+  for (int k = 0; k < K; k += 64) {
+    if (k + 32 < K) fetch(xb, wb, k + 32);
+    multiply(xa, wa);
+    if (k + 32 < K) {
+      if (k + 64 < K) fetch(xa, wa, k + 64);
+      multiply(xb, wb);
+    }
+  }
+  // acc[j][t][i] is the sum for row 16 t + r and column n0 + 16 (j & 1) + 4 g + i
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    if (16 * t + r >= rows) continue;
+    TO* orow = out + static_cast<size_t>(row0 + 16 * t + r) * ldo;
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int n = n0 + 16 * j + 4 * g + i;
+        if (n >= N) continue;
+        float v = acc[j][t][i];
+        if constexpr (GLU) v = v / (1.0f + expf(-v)) * acc[2 + j][t][i];
+        orow[n] = from_float<TO>(v);
+      }
+  }
+}
+
+static int grouped_checks(const char* name, const void* x, long long ldx, const void* w, long long ldw, int K, int N,
+                          int pairs, int n_experts) {
+  PYLON_REQUIRE(pairs >= 0 && n_experts >= 1 && N >= 1 && K >= 8 && K % 8 == 0,
+                "%s: rows of a multiple of 8 elements, got %d", name, K);
+  PYLON_REQUIRE(ldx % 8 == 0 && ldw % 8 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 &&
+                    reinterpret_cast<uintptr_t>(w) % 16 == 0,
+                "%s: rows must start at 16-byte aligned addresses", name);
+  PYLON_REQUIRE(ldx >= K && ldw >= K, "%s: rows overlap", name);
+  return 0;
+}
+
+// hidden[p] = silu(W_gate[e] x[row_index[p]]) * (W_up[e] x[row_index[p]]) for the sorted pairs p of
+// every expert e (offsets: int [n_experts + 1]); x bfloat16 [tokens, width]; w bfloat16
+// [n_experts * 2 ff, width]; hidden bfloat16 [pairs, ff].
+extern "C" int pylon_grouped_gate_up(void* hidden, const void* x, long long ldx, const int* row_index, const void* w,
+                                     long long ldw, const int* offsets, int pairs, int n_experts, int ff, int width,
+                                     hipStream_t stream) {
+  if (grouped_checks("grouped_gate_up", x, ldx, w, ldw, width, ff, pairs, n_experts)) return 1;
+  if (pairs == 0) return 0;
+  dim3 grid(pairs / MX_TM + n_experts, (ff + 4 * MX_WAVE_COLS - 1) / (4 * MX_WAVE_COLS)), block(256);
+  PYLON_REQUIRE(grid.y <= 65535, "grouped_gate_up: too many columns for one launch");
+  hipLaunchKernelGGL((grouped_rows_kernel<true, bf16_t>), grid, block, 0, stream, (bf16_t*)hidden, (long long)ff,
+                     (const uint16_t*)x, ldx, row_index, (const uint16_t*)w, ldw, 2ll * ff, offsets, n_experts, ff,
+                     width);
+  PYLON_LAUNCHED("grouped_gate_up");
+}
+
+// y[p] = W_down[e] hidden[p] for the sorted pairs p of every expert e: hidden bfloat16 [pairs, ff],
+// w bfloat16 [n_experts * width, ff], y float [pairs, width].
+extern "C" int pylon_grouped_down(float* y, const void* hidden, long long ldh, const void* w, long long ldw,
+                                  const int* offsets, int pairs, int n_experts, int ff, int width,
+                                  hipStream_t stream) {
+  if (grouped_checks("grouped_down", hidden, ldh, w, ldw, ff, width, pairs, n_experts)) return 1;
+  if (pairs == 0) return 0;
+  dim3 grid(pairs / MX_TM + n_experts, (width + 4 * MX_WAVE_COLS - 1) / (4 * MX_WAVE_COLS)), block(256);
+  PYLON_REQUIRE(grid.y <= 65535, "grouped_down: too many columns for one launch");
+  hipLaunchKernelGGL((grouped_rows_kernel<false, float>), grid, block, 0, stream, y, (long long)width,
+                     (const uint16_t*)hidden, ldh, nullptr, (const uint16_t*)w, ldw, (long long)width, offsets,
+                     n_experts, width, ff);
+  PYLON_LAUNCHED("grouped_down");
+}
+
+__global__ void __launch_bounds__(256)
+expert_combine_kernel(float* __restrict__ out, const float* __restrict__ y, const int* __restrict__ place,
+                      const float* __restrict__ weights, const float* __restrict__ shared,
+                      const float* __restrict__ shared_gate, int top, int width) {
+  const int t = blockIdx.y;
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= width) return;
+  float acc = 0.f;
+  for (int s = 0; s < top; ++s)
+    acc = fmaf(weights[static_cast<size_t>(t) * top + s], y[static_cast<size_t>(place[static_cast<size_t>(t) * top + s]) * width + c], acc);
+  if (shared != nullptr) acc = fmaf(shared_gate != nullptr ? shared_gate[t] : 1.f, shared[static_cast<size_t>(t) * width + c], acc);
+  out[static_cast<size_t>(t) * width + c] = acc;
+}
+
+// out[t] = sum_s weights[t, s] y[place[t, s]] (+ shared_gate[t] * shared[t]): the experts' outputs of
+// the sorted pairs brought back to their tokens, in the order of the token's choices.
+extern "C" int pylon_expert_combine(float* out, const float* y, const int* place, const float* weights,
+                                    const float* shared, const float* shared_gate, int tokens, int top, int width,
+                                    hipStream_t stream) {
+  PYLON_REQUIRE(tokens >= 0 && top >= 1 && width >= 1, "expert_combine: sizes must be positive");
+  if (tokens == 0) return 0;
+  for (int first = 0; first < tokens; first += 65535) {
+    const int n = tokens - first < 65535 ? tokens - first : 65535;
+    const size_t off = static_cast<size_t>(first);
+    hipLaunchKernelGGL(expert_combine_kernel, dim3((width + 255) / 256, n), dim3(256), 0, stream, out + off * width, y,
+                       place + off * top, weights + off * top, shared != nullptr ? shared + off * width : nullptr,
+                       shared_gate != nullptr ? shared_gate + off : nullptr, top, width);
+  }
+  PYLON_LAUNCHED("expert_combine");
+}

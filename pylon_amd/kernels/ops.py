@@ -1185,6 +1185,52 @@ def expert_down(hidden: torch.Tensor, down: torch.Tensor, experts: torch.Tensor,
     return out
 
 
+GROUPED_FROM = 33  # from this many tokens of a step on, the experts' products run expert by expert on the matrix cores
+
+
+def experts_grouped_ok(x: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor) -> bool:
+    """Whether :func:`experts_grouped` takes these operands: bfloat16 throughout, rows of multiples
+    of 8 elements at 16-byte aligned addresses."""
+    return (x.dtype == torch.bfloat16 and gate_up.dtype == torch.bfloat16 and down.dtype == torch.bfloat16
+            and x.shape[1] % 8 == 0 and down.shape[1] % 8 == 0 and x.stride(0) % 8 == 0 and x.stride(1) == 1
+            and gate_up.stride(0) % 8 == 0 and down.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0
+            and gate_up.data_ptr() % 16 == 0 and down.data_ptr() % 16 == 0)
+
+
+def experts_grouped(x: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, experts: torch.Tensor,
+                    weights: torch.Tensor, *, n_experts: int, ff: int, shared: Optional[torch.Tensor] = None,
+                    shared_gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """What :func:`expert_gate_up` and :func:`expert_down` compute, for many bfloat16 tokens: the
+    (token, choice) pairs are sorted by expert on the device (nothing is read back), every expert's
+    pairs go through its gate/up and its down matrix as tiles of 64 rows on the matrix cores, and
+    the results return to their tokens weighted, in the order of the token's choices.  float32
+    ``[tokens, width]``."""
+    tokens, width = x.shape
+    top = experts.shape[1]
+    pairs = tokens * top
+    if not experts_grouped_ok(x, gate_up, down):
+        raise KernelError("experts_grouped does not take these operands")
+    if gate_up.shape != (n_experts * 2 * ff, width) or down.shape != (n_experts * width, ff):
+        raise KernelError("experts_grouped: the experts' matrices must be [experts * 2 ff, width] and [experts * width, ff]")
+    flat = experts.reshape(-1).long()
+    order = torch.argsort(flat, stable=True)  # sorted place -> pair
+    bounds = torch.arange(n_experts + 1, device=x.device)
+    offsets = torch.searchsorted(flat[order], bounds).to(torch.int32)
+    rows = (order // top).to(torch.int32)  # sorted place -> token
+    place = torch.empty_like(order).scatter_(0, order, torch.arange(pairs, device=x.device)).to(torch.int32)
+    hidden = torch.empty((pairs, ff), dtype=torch.bfloat16, device=x.device)
+    _lib.call("pylon_grouped_gate_up", _dev(hidden, "hidden"), x.data_ptr(), x.stride(0), _dev(rows, "rows"),
+              gate_up.data_ptr(), gate_up.stride(0), _dev(offsets, "offsets"), pairs, n_experts, ff, width, _stream())
+    y = torch.empty((pairs, width), dtype=torch.float32, device=x.device)
+    _lib.call("pylon_grouped_down", _dev(y, "y"), _dev(hidden, "hidden"), ff, down.data_ptr(), down.stride(0),
+              _dev(offsets, "offsets"), pairs, n_experts, ff, width, _stream())
+    out = torch.empty((tokens, width), dtype=torch.float32, device=x.device)
+    _lib.call("pylon_expert_combine", _dev(out, "out"), _dev(y, "y"), _dev(place, "place"),
+              _dev(weights, "weights", torch.float32), _dev(shared, "shared", torch.float32),
+              _dev(shared_gate, "shared_gate", torch.float32), tokens, top, width, _stream())
+    return out
+
+
 def probe_read(data: torch.Tensor, sink: torch.Tensor) -> None:
     """Read every byte of ``data`` once (a measurement aid: the device's read bandwidth)."""
     if not data.is_contiguous() or not data.is_cuda:

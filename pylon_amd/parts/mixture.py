@@ -5,7 +5,8 @@ the model's type; with a gated shared expert its gate vector is one more row of 
 one kernel picks every token's ``top`` experts and the softmax over their logits; one computes
 ``silu(gate) * up`` of every (token, chosen expert) from the experts' fused gate/up matrix, and one
 applies the chosen experts' down matrices, weights the results and adds the shared expert's output
-times its gate.  The shared expert itself is an ordinary gated feed-forward on the engine's
+times its gate (from 33 bfloat16 tokens on, the (token, expert) pairs are sorted by expert on the
+device instead and every expert's pairs run as tiles on the matrix cores).  The shared expert itself is an ordinary gated feed-forward on the engine's
 product kernels.  The result is float32 and goes to the residual sum unrounded.  A token's
 output does not depend on which other tokens share its step: every kernel here works token by
 token with a fixed order of additions.
@@ -51,11 +52,16 @@ class MixtureFeedForward(Part):
         experts, weights, shared_gate = ops.route_top(
             logits, self.params.get("router_bias"), n_experts=spec.n_experts, top=spec.top,
             shared_gate=spec.shared_gate)
-        hidden = ops.expert_gate_up(h, self.params["gate_up"], experts, n_experts=spec.n_experts, ff=spec.expert_size)
         shared = None
         if spec.shared_size is not None:
             shared_hidden = ops.linear_glu(h, self.params["shared_gate_up"], out_dtype=self.dtype)
             shared = ops.linear(shared_hidden, self.params["shared_down"], out_dtype=torch.float32)
+        if h.shape[0] >= ops.GROUPED_FROM and ops.experts_grouped_ok(h, self.params["gate_up"], self.params["down"]):
+            # many tokens: sorted by expert, every expert's tokens as tiles on the matrix cores
+            return ops.experts_grouped(h, self.params["gate_up"], self.params["down"], experts, weights,
+                                       n_experts=spec.n_experts, ff=spec.expert_size, shared=shared,
+                                       shared_gate=shared_gate)
+        hidden = ops.expert_gate_up(h, self.params["gate_up"], experts, n_experts=spec.n_experts, ff=spec.expert_size)
         return ops.expert_down(hidden, self.params["down"], experts, weights, n_experts=spec.n_experts,
                                width=spec.hidden_size, shared=shared, shared_gate=shared_gate)
 
