@@ -8,8 +8,8 @@
 //   the normed query latent, the normed key/value latent into its cache slot, and sigmoid of the
 //   gate logits.  Norms (root mean square, eps inside the root, times a weight) in float.
 // head_project: out[t, h, :] = gate[t, h] * x[t, h, :] @ m[h] with m [heads, n_in, n_out]; a
-//   workgroup keeps the inputs of a few tokens in LDS and walks m[h] once for all of them; sums
-//   in float in the order of n_in, whatever the batch.
+//   workgroup keeps the inputs of a few tokens in LDS and walks 64 columns of m[h] once for all of
+//   them, its four waves a quarter of n_in each; sums in float in one fixed order, whatever the batch.
 // gate_heads: x[t, h, :] *= gate[t, h] in place.
 #include "common.h"
 
@@ -67,12 +67,15 @@ extern "C" int pylon_latent_prepare(void* q_latent, void* c_cache, float* gate_o
 
 #define HP_THREADS 256
 #define HP_TOKENS 8
+#define HP_COLS 64   // outputs of a workgroup
+#define HP_SLICES 4  // the waves of a workgroup cut n_in between them
 
 template <typename TX, typename TM>
 __global__ void __launch_bounds__(HP_THREADS)
 head_project_kernel(TX* __restrict__ out, const TX* __restrict__ x, long long x_stride, const TM* __restrict__ m,
                     const float* __restrict__ gate, int tokens, int heads, int n_in, int n_out) {
-  extern __shared__ float xs[];  // [HP_TOKENS, n_in]
+  extern __shared__ float xs[];  // [HP_TOKENS, n_in], then the slices' partial sums [HP_SLICES, HP_TOKENS, HP_COLS]
+  float* partial = xs + HP_TOKENS * n_in;
   const int t0 = blockIdx.x * HP_TOKENS, h = blockIdx.y, tid = threadIdx.x;
   for (int i = tid; i < HP_TOKENS * n_in; i += HP_THREADS) {
     const int tt = i / n_in, k = i - tt * n_in;
@@ -80,23 +83,34 @@ head_project_kernel(TX* __restrict__ out, const TX* __restrict__ x, long long x_
                                : 0.f;
   }
   __syncthreads();
-  const TM* mh = m + static_cast<size_t>(h) * n_in * n_out;
-  for (int o = blockIdx.z * HP_THREADS + tid; o < n_out; o += gridDim.z * HP_THREADS) {
-    float acc[HP_TOKENS];
+  const int slice = tid / HP_COLS, col = tid % HP_COLS;
+  const int o = blockIdx.z * HP_COLS + col;
+  const int per = (n_in + HP_SLICES - 1) / HP_SLICES;
+  const int k0 = slice * per, k1 = k0 + per < n_in ? k0 + per : n_in;
+  float acc[HP_TOKENS];
 #pragma unroll
-    for (int tt = 0; tt < HP_TOKENS; ++tt) acc[tt] = 0.f;
-    for (int k = 0; k < n_in; ++k) {
-      const float w = to_float(mh[static_cast<size_t>(k) * n_out + o]);
+  for (int tt = 0; tt < HP_TOKENS; ++tt) acc[tt] = 0.f;
+  if (o < n_out) {
+    const TM* mh = m + static_cast<size_t>(h) * n_in * n_out + o;
+    for (int k = k0; k < k1; ++k) {
+      const float w = to_float(mh[static_cast<size_t>(k) * n_out]);
 #pragma unroll
       for (int tt = 0; tt < HP_TOKENS; ++tt) acc[tt] = fmaf(xs[tt * n_in + k], w, acc[tt]);
     }
+  }
 #pragma unroll
-    for (int tt = 0; tt < HP_TOKENS; ++tt) {
-      if (t0 + tt < tokens) {
-        const float g = gate != nullptr ? gate[static_cast<size_t>(t0 + tt) * heads + h] : 1.f;
-        out[(static_cast<size_t>(t0 + tt) * heads + h) * n_out + o] = from_float<TX>(acc[tt] * g);
-      }
-    }
+  for (int tt = 0; tt < HP_TOKENS; ++tt) partial[(slice * HP_TOKENS + tt) * HP_COLS + col] = acc[tt];
+  __syncthreads();
+  // the slices' sums are added in their order, whatever the batch
+  for (int i = tid; i < HP_TOKENS * HP_COLS; i += HP_THREADS) {
+    const int tt = i / HP_COLS, c = i % HP_COLS;
+    const int oc = blockIdx.z * HP_COLS + c;
+    if (t0 + tt >= tokens || oc >= n_out) continue;
+    float sum = partial[tt * HP_COLS + c];
+#pragma unroll
+    for (int sl = 1; sl < HP_SLICES; ++sl) sum += partial[(sl * HP_TOKENS + tt) * HP_COLS + c];
+    const float g = gate != nullptr ? gate[static_cast<size_t>(t0 + tt) * heads + h] : 1.f;
+    out[(static_cast<size_t>(t0 + tt) * heads + h) * n_out + oc] = from_float<TX>(sum * g);
   }
 }
 
@@ -109,12 +123,12 @@ extern "C" int pylon_head_project(void* out, const void* x, int x_dtype, long lo
   PYLON_REQUIRE(tokens >= 0 && heads > 0 && n_in > 0 && n_out > 0, "head_project: sizes must be positive");
   PYLON_REQUIRE(heads <= 65535, "head_project: too many heads for one launch");
   PYLON_REQUIRE(x_stride >= static_cast<long long>(heads) * n_in, "head_project: rows of x overlap");
-  const size_t lds = sizeof(float) * HP_TOKENS * n_in;
+  const size_t lds = sizeof(float) * (HP_TOKENS * n_in + HP_SLICES * HP_TOKENS * HP_COLS);
   PYLON_REQUIRE(lds <= 64 * 1024, "head_project: %d inputs per head do not fit LDS", n_in);
   PYLON_REQUIRE(!(x_dtype == PYLON_F32 && m_dtype == PYLON_BF16), "head_project: float inputs take a float matrix");
   if (tokens == 0) return 0;
-  int zs = (n_out + HP_THREADS - 1) / HP_THREADS;
-  if (zs > 64) zs = 64;
+  const int zs = (n_out + HP_COLS - 1) / HP_COLS;
+  PYLON_REQUIRE(zs <= 65535, "head_project: too many outputs per head for one launch");
   dim3 grid((tokens + HP_TOKENS - 1) / HP_TOKENS, heads, zs), block(HP_THREADS);
 #define GO(TX, TM)                                                                                              \
   hipLaunchKernelGGL((head_project_kernel<TX, TM>), grid, block, lds, stream, (TX*)out, (const TX*)x, x_stride, \

@@ -297,8 +297,7 @@ def weight_targets(cfg: PavitarConfig) -> Dict[str, WeightTarget]:
         if layer.mlp is not None:
             mlp, ff = layer.mlp, layer.mlp.ff
             targets[f"{src}.norm2"] = WeightTarget(f"{dst}.feed_forward_norm.weight", (width,), **around_zero)
-            targets[f"{src}.mlp.router"] = WeightTarget(f"{dst}.feed_forward.router", (mlp.experts, width), 0,
-                                                        role="vector")
+            targets[f"{src}.mlp.router"] = WeightTarget(f"{dst}.feed_forward.router", (mlp.experts, width), 0)
             targets[f"{src}.mlp.router.b"] = WeightTarget(f"{dst}.feed_forward.router_bias", (mlp.experts,),
                                                           role="vector", init="normal")
             for e in range(mlp.experts):
@@ -310,8 +309,7 @@ def weight_targets(cfg: PavitarConfig) -> Dict[str, WeightTarget]:
                 targets[f"{src}.mlp.shared.gate"] = WeightTarget(f"{dst}.feed_forward.shared_gate_up", (sff, width), 0)
                 targets[f"{src}.mlp.shared.up"] = WeightTarget(f"{dst}.feed_forward.shared_gate_up", (sff, width), sff)
                 targets[f"{src}.mlp.shared.down"] = WeightTarget(f"{dst}.feed_forward.shared_down", (width, sff))
-                targets[f"{src}.mlp.shared.sg"] = WeightTarget(f"{dst}.feed_forward.router", (1, width), mlp.experts,
-                                                               role="vector")
+                targets[f"{src}.mlp.shared.sg"] = WeightTarget(f"{dst}.feed_forward.router", (1, width), mlp.experts)
     return targets
 
 

@@ -72,6 +72,16 @@ class LatentAttention(Part):
         limit = self.spec.window if self.spec.window is not None else self.spec.chunk
         return bound if limit is None else min(bound, limit)
 
+    def _decode_launch(self, queries: int, span: int) -> tuple:
+        """(cuts, waves) of the decode kernel for ``queries`` query tokens (a group of heads each) over
+        one shared key/value head: with so few workgroups a request's latents are cut over workgroups
+        down to 128 a cut, until the workgroups fill the chip."""
+        units = ops.compute_units()
+        cuts = 1
+        while cuts < 64 and queries * cuts * 2 <= units and cuts * 2 * 128 <= span:
+            cuts *= 2
+        return cuts, ops.decode_splits(queries * cuts, 1, -(-span // cuts), units)
+
     def _matrix_cores(self) -> bool:
         return self.dtype == torch.bfloat16 and self.spec.kv_rank in ops.DECODE_HEAD_DIMS
 
@@ -79,7 +89,7 @@ class LatentAttention(Part):
         if not self._matrix_cores():
             return ("latent_attention",)
         group = head_group(self.spec.n_heads)
-        return ("latent_attention",) + tuple(ops.decode_launch(rows * (self.spec.n_heads // group), 1, self._span(bound)))
+        return ("latent_attention",) + tuple(self._decode_launch(rows * (self.spec.n_heads // group), self._span(bound)))
 
     def forward(self, h: torch.Tensor, ctx, cache, stores: bool) -> torch.Tensor:
         spec = self.spec
@@ -102,7 +112,7 @@ class LatentAttention(Part):
             if repeat > 1:  # every group of heads a query token of its own, on its request's row of the table
                 positions = ctx.positions.repeat_interleave(repeat)
                 rows = ctx.tok_row.repeat_interleave(repeat)
-            cuts, splits = ops.decode_launch(tokens * repeat, 1, self._span(ctx.max_len))
+            cuts, splits = self._decode_launch(tokens * repeat, self._span(ctx.max_len))
             mixed = ops.attention_decode(
                 q.view(tokens * repeat, group, rank), latents, latents, cache.block_table, rows, positions,
                 page_size=cache.page_size, scale=spec.scale, n_splits=splits, n_cuts=cuts, **mask,

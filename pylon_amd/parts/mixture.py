@@ -1,7 +1,9 @@
 """A mixture of gated feed-forward experts with an optional shared expert.
 
-Router logits ``W_r h + b`` are a float32 product (the router's matrix is kept in float32 whatever
-the model's type; with a gated shared expert its gate vector is one more row of the same matrix);
+Router logits ``W_r h + b`` are float32 sums of exact products (``ops.linear`` with a float32
+result: bfloat16 operands on the matrix cores with float32 accumulation, never rounded; float32
+operands on the exact kernel; with a gated shared expert its gate vector is one more row of the
+router's matrix);
 one kernel picks every token's ``top`` experts and the softmax over their logits; one computes
 ``silu(gate) * up`` of every (token, chosen expert) from the experts' fused gate/up matrix, and one
 applies the chosen experts' down matrices, weights the results and adds the shared expert's output
@@ -34,7 +36,9 @@ class MixtureFeedForward(Part):
         self.dtype = dtype
         width, ff = spec.hidden_size, spec.expert_size
         self.router_rows = spec.n_experts + (1 if spec.shared_gate else 0)
-        self.add_param("router", (self.router_rows, width), torch.float32, device, role="vector")
+        # stored in 16 bits it stays so: products of two bfloat16 numbers are exact in float32, and the
+        # product kernels add them up in float32 and hand the sums back unrounded
+        self.add_param("router", (self.router_rows, width), dtype, device)
         if spec.router_bias:
             self.add_param("router_bias", (spec.n_experts,), torch.float32, device, role="vector")
         # expert e: rows [e * 2 ff, e * 2 ff + ff) its gate, the next ff its up; rows [e * width, ...) its down
@@ -48,7 +52,7 @@ class MixtureFeedForward(Part):
 
     def forward(self, h: torch.Tensor, ctx) -> torch.Tensor:
         spec = self.spec
-        logits = ops.gemm_tiled(h, self.params["router"], out_dtype=torch.float32)
+        logits = ops.linear(h, self.params["router"], out_dtype=torch.float32)
         experts, weights, shared_gate = ops.route_top(
             logits, self.params.get("router_bias"), n_experts=spec.n_experts, top=spec.top,
             shared_gate=spec.shared_gate)

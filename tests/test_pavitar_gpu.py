@@ -270,14 +270,14 @@ def test_mixture_of_experts_against_the_plain_one(ops, dtype, width, experts, to
         w["f.shared.down"], w["f.shared.sg"] = rng.normal(size=(width, shared)) * 0.2, rng.normal(size=(1, width)) * 0.3
     w = {k: torch.tensor(a).to(dtype).double().numpy() for k, a in w.items()}  # what the part will hold
     p = part.params
-    p["router"][:experts] = dev(w["f.router"])
+    p["router"][:experts] = dev(w["f.router"], dtype)
     p["router_bias"][:] = dev(w["f.router.b"])
     for e in range(experts):
         p["gate_up"][e * 2 * ff: e * 2 * ff + ff] = dev(w[f"f.e{e}.gate"], dtype)
         p["gate_up"][e * 2 * ff + ff: (e + 1) * 2 * ff] = dev(w[f"f.e{e}.up"], dtype)
         p["down"][e * width: (e + 1) * width] = dev(w[f"f.e{e}.down"], dtype)
     if shared is not None:
-        p["router"][experts:] = dev(w["f.shared.sg"])
+        p["router"][experts:] = dev(w["f.shared.sg"], dtype)
         p["shared_gate_up"][:shared] = dev(w["f.shared.gate"], dtype)
         p["shared_gate_up"][shared:] = dev(w["f.shared.up"], dtype)
         p["shared_down"][:] = dev(w["f.shared.down"], dtype)
