@@ -92,7 +92,8 @@ head_project_kernel(TX* __restrict__ out, const TX* __restrict__ x, long long x_
   for (int tt = 0; tt < HP_TOKENS; ++tt) acc[tt] = 0.f;
   if (o < n_out) {
     const TM* mh = m + static_cast<size_t>(h) * n_in * n_out + o;
-    for (int k = k0; k < k1; ++k) {
+#pragma unroll 8
+    for (int k = k0; k < k1; ++k) {  // unrolled: eight loads of m in flight
       const float w = to_float(mh[static_cast<size_t>(k) * n_out]);
 #pragma unroll
       for (int tt = 0; tt < HP_TOKENS; ++tt) acc[tt] = fmaf(xs[tt * n_in + k], w, acc[tt]);

@@ -259,8 +259,9 @@ extern "C" int pylon_expert_down(float* out, const void* hidden, int h_dtype, co
 
 // ---- many tokens: the experts' products on the matrix cores, expert by expert ------------------
 // The (token, choice) pairs are sorted by expert (on the device, by the caller); offsets[e] is the
-// first sorted pair of expert e.  A workgroup takes 64 sorted pairs of one expert and 128 output
-// columns: four waves of 32 columns each, all 64 rows, operands fetched in the shape the matrix
+// first sorted pair of expert e.  A workgroup takes 64 or 128 sorted pairs of one expert (128 where
+// the experts have that many on average: the larger tile re-reads the weights half as often) and
+// 128 output columns: four waves of 32 columns each, all rows, operands fetched in the shape the matrix
 // instruction wants them (a lane: 8 neighbouring elements of one row), the next 32 elements of
 // K in flight while the current ones are multiplied.  Which (expert, rows) a workgroup has it
 // finds from the offsets itself; the grid is the most tiles there can be, and the workgroups
@@ -269,14 +270,14 @@ extern "C" int pylon_expert_down(float* out, const void* hidden, int h_dtype, co
 typedef __bf16 mx_bf16x8 __attribute__((ext_vector_type(8)));
 typedef float mx_floatx4 __attribute__((ext_vector_type(4)));
 
-#define MX_TM 64
 #define MX_WAVE_COLS 32
 
-template <bool GLU, typename TO>
+template <bool GLU, int MT, typename TO>
 __global__ void __launch_bounds__(256)
 grouped_rows_kernel(TO* __restrict__ out, long long ldo, const uint16_t* __restrict__ x, long long ldx,
                     const int* __restrict__ row_index, const uint16_t* __restrict__ w, long long ldw,
                     long long expert_rows, const int* __restrict__ offsets, int n_experts, int N, int K) {
+  constexpr int MX_TM = 16 * MT;  // rows of a tile
   constexpr int J = GLU ? 4 : 2;  // weight tiles of a wave: GLU: two of gate rows, then the two of their up rows
   const int lane = threadIdx.x & (PYLON_WAVE - 1), wave = threadIdx.x / PYLON_WAVE;
   const int r = lane & 15, g = lane >> 4;
@@ -296,9 +297,9 @@ grouped_rows_kernel(TO* __restrict__ out, long long ldo, const uint16_t* __restr
   const int n0 = blockIdx.y * (4 * MX_WAVE_COLS) + wave * MX_WAVE_COLS;
   if (n0 >= N) return;
 
-  const uint16_t* xp[4];
+  const uint16_t* xp[MT];
 #pragma unroll
-  for (int t = 0; t < 4; ++t) {
+  for (int t = 0; t < MT; ++t) {
     const int local = 16 * t + r < rows ? 16 * t + r : 0;  // rows past the tile's last repeat its first
     const int m = row0 + local;
     xp[t] = x + static_cast<size_t>(row_index != nullptr ? row_index[m] : m) * ldx + 8 * g;
@@ -311,27 +312,27 @@ grouped_rows_kernel(TO* __restrict__ out, long long ldo, const uint16_t* __restr
     const size_t row = static_cast<size_t>(e) * expert_rows + (GLU && j >= 2 ? N : 0) + n;
     wp[j] = w + row * ldw + 8 * g;
   }
-  mx_floatx4 acc[J][4];
+  mx_floatx4 acc[J][MT];
 #pragma unroll
   for (int j = 0; j < J; ++j)
 #pragma unroll
-    for (int t = 0; t < 4; ++t) acc[j][t] = mx_floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int t = 0; t < MT; ++t) acc[j][t] = mx_floatx4{0.f, 0.f, 0.f, 0.f};
 
   const mx_bf16x8 zero = __builtin_bit_cast(mx_bf16x8, uint4{0u, 0u, 0u, 0u});
-  auto fetch = [&](mx_bf16x8(&xa)[4], mx_bf16x8(&wa)[J], int k) {
+  auto fetch = [&](mx_bf16x8(&xa)[MT], mx_bf16x8(&wa)[J], int k) {
     const bool ok = k + 8 * g < K;  // K is a multiple of 8: a lane's 8 elements are all inside or all outside
 #pragma unroll
-    for (int t = 0; t < 4; ++t) xa[t] = ok ? *reinterpret_cast<const mx_bf16x8*>(xp[t] + k) : zero;
+    for (int t = 0; t < MT; ++t) xa[t] = ok ? *reinterpret_cast<const mx_bf16x8*>(xp[t] + k) : zero;
 #pragma unroll
     for (int j = 0; j < J; ++j) wa[j] = ok ? *reinterpret_cast<const mx_bf16x8*>(wp[j] + k) : zero;
   };
-  auto multiply = [&](const mx_bf16x8(&xa)[4], const mx_bf16x8(&wa)[J]) {
+  auto multiply = [&](const mx_bf16x8(&xa)[MT], const mx_bf16x8(&wa)[J]) {
 #pragma unroll
     for (int j = 0; j < J; ++j)
 #pragma unroll
-      for (int t = 0; t < 4; ++t) acc[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[j], xa[t], acc[j][t], 0, 0, 0);
+      for (int t = 0; t < MT; ++t) acc[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[j], xa[t], acc[j][t], 0, 0, 0);
   };
-  mx_bf16x8 xa[4], wa[J], xb[4], wb[J];
+  mx_bf16x8 xa[MT], wa[J], xb[MT], wb[J];
   fetch(xa, wa, 0);
   for (int k = 0; k < K; k += 64) {
     if (k + 32 < K) fetch(xb, wb, k + 32);
@@ -343,7 +344,7 @@ grouped_rows_kernel(TO* __restrict__ out, long long ldo, const uint16_t* __restr
   }
   // acc[j][t][i] is the sum for row 16 t + r and column n0 + 16 (j & 1) + 4 g + i
 #pragma unroll
-  for (int t = 0; t < 4; ++t) {
+  for (int t = 0; t < MT; ++t) {
     if (16 * t + r >= rows) continue;
     TO* orow = out + static_cast<size_t>(row0 + 16 * t + r) * ldo;
 #pragma unroll
@@ -359,6 +360,119 @@ grouped_rows_kernel(TO* __restrict__ out, long long ldo, const uint16_t* __restr
   }
 }
 
+// The same product for experts with many pairs each: tiles of 128 pairs x 128 output columns
+// (with the gated epilogue: 128 gate and their 128 up columns), K in pieces of 64 elements that all
+// 256 threads bring into LDS together, whole 128-byte row segments at a time (a thread 16 bytes of
+// one row; 32 rows further on its next load), the next piece on its way into registers while the
+// matrix instructions read the current one from LDS.  Rows lie 144 bytes apart in LDS, so that
+// the 16 rows of an operand fall into different banks.  A wave takes all 128 rows and 32 columns.
+#define GT_ROWS 128
+#define GT_COLS 128
+#define GT_K 64
+#define GT_PITCH 144
+
+template <bool GLU, typename TO>
+__global__ void __launch_bounds__(256)
+grouped_tiles_kernel(TO* __restrict__ out, long long ldo, const uint16_t* __restrict__ x, long long ldx,
+                     const int* __restrict__ row_index, const uint16_t* __restrict__ w, long long ldw,
+                     long long expert_rows, const int* __restrict__ offsets, int n_experts, int N, int K) {
+  constexpr int WROWS = GLU ? 2 * GT_COLS : GT_COLS;
+  constexpr int XLOADS = GT_ROWS / 32, LOADS = (GT_ROWS + WROWS) / 32;
+  constexpr int J = GLU ? 4 : 2, MT = GT_ROWS / 16;
+  __shared__ __attribute__((aligned(16))) unsigned char lds[(GT_ROWS + WROWS) * GT_PITCH];
+  const int tid = threadIdx.x, lane = tid & (PYLON_WAVE - 1), wave = tid / PYLON_WAVE;
+  const int r = lane & 15, g = lane >> 4;
+  int tile = blockIdx.x, e = 0, row0 = 0, rows = 0;
+  for (; e < n_experts; ++e) {
+    const int begin = offsets[e], count = offsets[e + 1] - begin;
+    const int tiles = (count + GT_ROWS - 1) / GT_ROWS;
+    if (tile < tiles) {
+      row0 = begin + tile * GT_ROWS;
+      rows = count - tile * GT_ROWS < GT_ROWS ? count - tile * GT_ROWS : GT_ROWS;
+      break;
+    }
+    tile -= tiles;
+  }
+  if (e == n_experts) return;  // the whole workgroup: no barrier is missed
+  const int n0 = blockIdx.y * GT_COLS;
+
+  // what this thread brings: the 16-byte piece `piece` of rows lrow, lrow + 32, ... of the tile in LDS
+  const int piece = tid & 7, lrow = tid >> 3;
+  unsigned src[LOADS];  // in elements, from x (the first XLOADS) or from w
+#pragma unroll
+  for (int i = 0; i < LOADS; ++i) {
+    const int row = lrow + 32 * i;
+    if (i < XLOADS) {
+      const int m = row0 + (row < rows ? row : 0);  // rows past the tile's last repeat its first
+      src[i] = static_cast<unsigned>((row_index != nullptr ? row_index[m] : m) * ldx + piece * 8);
+    } else {
+      const int c = row - GT_ROWS;
+      const bool up = GLU && c >= GT_COLS;
+      int n = n0 + (up ? c - GT_COLS : c);
+      if (n >= N) n = N - 1;  // columns past the last repeat it; they are not stored
+      src[i] = static_cast<unsigned>((e * expert_rows + (up ? N : 0) + n) * ldw + piece * 8);
+    }
+  }
+  uint4 held[LOADS];
+  auto fetch = [&](int k) {
+    const bool ok = k + piece * 8 < K;  // K is a multiple of 8
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i)
+      held[i] = ok ? *reinterpret_cast<const uint4*>((i < XLOADS ? x : w) + src[i] + k) : uint4{0u, 0u, 0u, 0u};
+  };
+  mx_floatx4 acc[J][MT];
+#pragma unroll
+  for (int j = 0; j < J; ++j)
+#pragma unroll
+    for (int t = 0; t < MT; ++t) acc[j][t] = mx_floatx4{0.f, 0.f, 0.f, 0.f};
+
+  fetch(0);
+  for (int k = 0; k < K; k += GT_K) {
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i) *reinterpret_cast<uint4*>(lds + (lrow + 32 * i) * GT_PITCH + piece * 16) = held[i];
+    __syncthreads();
+    if (k + GT_K < K) fetch(k + GT_K);
+#pragma unroll
+    for (int h = 0; h < GT_K / 32; ++h) {
+      mx_bf16x8 wf[J];
+#pragma unroll
+      for (int j = 0; j < J; ++j) {
+        const int row = GT_ROWS + (GLU && j >= 2 ? GT_COLS : 0) + wave * 32 + 16 * (j & 1) + r;
+        wf[j] = *reinterpret_cast<const mx_bf16x8*>(lds + row * GT_PITCH + h * 64 + g * 16);
+      }
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        const mx_bf16x8 xf = *reinterpret_cast<const mx_bf16x8*>(lds + (16 * t + r) * GT_PITCH + h * 64 + g * 16);
+#pragma unroll
+        for (int j = 0; j < J; ++j) acc[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[j], xf, acc[j][t], 0, 0, 0);
+      }
+    }
+    __syncthreads();
+  }
+  // acc[j][t][i] is the sum for row 16 t + r and column n0 + 32 wave + 16 (j & 1) + 4 g + i
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    if (16 * t + r >= rows) continue;
+    TO* orow = out + static_cast<size_t>(row0 + 16 * t + r) * ldo;
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int n = n0 + 32 * wave + 16 * j + 4 * g + i;
+        if (n >= N) continue;
+        float v = acc[j][t][i];
+        if constexpr (GLU) v = v / (1.0f + expf(-v)) * acc[2 + j][t][i];
+        orow[n] = from_float<TO>(v);
+      }
+  }
+}
+
+// Tiles of 128 pairs through LDS pay once the experts have that many pairs on average; their
+// 32-bit offsets must span both operands.
+static bool grouped_large(int pairs, int n_experts, long long x_elements, long long w_elements) {
+  return pairs / n_experts >= GT_ROWS && x_elements < (1ll << 32) && w_elements < (1ll << 32);
+}
+
 static int grouped_checks(const char* name, const void* x, long long ldx, const void* w, long long ldw, int K, int N,
                           int pairs, int n_experts) {
   PYLON_REQUIRE(pairs >= 0 && n_experts >= 1 && N >= 1 && K >= 8 && K % 8 == 0,
@@ -372,17 +486,24 @@ static int grouped_checks(const char* name, const void* x, long long ldx, const 
 
 // hidden[p] = silu(W_gate[e] x[row_index[p]]) * (W_up[e] x[row_index[p]]) for the sorted pairs p of
 // every expert e (offsets: int [n_experts + 1]); x bfloat16 [tokens, width]; w bfloat16
-// [n_experts * 2 ff, width]; hidden bfloat16 [pairs, ff].
+// [n_experts * 2 ff, width]; hidden bfloat16 [pairs, ff]; tokens_bound: the rows of x.
 extern "C" int pylon_grouped_gate_up(void* hidden, const void* x, long long ldx, const int* row_index, const void* w,
                                      long long ldw, const int* offsets, int pairs, int n_experts, int ff, int width,
-                                     hipStream_t stream) {
+                                     int tokens_bound, hipStream_t stream) {
   if (grouped_checks("grouped_gate_up", x, ldx, w, ldw, width, ff, pairs, n_experts)) return 1;
   if (pairs == 0) return 0;
-  dim3 grid(pairs / MX_TM + n_experts, (ff + 4 * MX_WAVE_COLS - 1) / (4 * MX_WAVE_COLS)), block(256);
+  const bool large = grouped_large(pairs, n_experts, tokens_bound * ldx, 2ll * n_experts * ff * ldw);
+  const int tile = large ? GT_ROWS : 64;
+  dim3 grid(pairs / tile + n_experts, (ff + 4 * MX_WAVE_COLS - 1) / (4 * MX_WAVE_COLS)), block(256);
   PYLON_REQUIRE(grid.y <= 65535, "grouped_gate_up: too many columns for one launch");
-  hipLaunchKernelGGL((grouped_rows_kernel<true, bf16_t>), grid, block, 0, stream, (bf16_t*)hidden, (long long)ff,
-                     (const uint16_t*)x, ldx, row_index, (const uint16_t*)w, ldw, 2ll * ff, offsets, n_experts, ff,
-                     width);
+  if (large)
+    hipLaunchKernelGGL((grouped_tiles_kernel<true, bf16_t>), grid, block, 0, stream, (bf16_t*)hidden, (long long)ff,
+                       (const uint16_t*)x, ldx, row_index, (const uint16_t*)w, ldw, 2ll * ff, offsets, n_experts, ff,
+                       width);
+  else
+    hipLaunchKernelGGL((grouped_rows_kernel<true, 4, bf16_t>), grid, block, 0, stream, (bf16_t*)hidden,
+                       (long long)ff, (const uint16_t*)x, ldx, row_index, (const uint16_t*)w, ldw, 2ll * ff, offsets,
+                       n_experts, ff, width);
   PYLON_LAUNCHED("grouped_gate_up");
 }
 
@@ -393,11 +514,18 @@ extern "C" int pylon_grouped_down(float* y, const void* hidden, long long ldh, c
                                   hipStream_t stream) {
   if (grouped_checks("grouped_down", hidden, ldh, w, ldw, ff, width, pairs, n_experts)) return 1;
   if (pairs == 0) return 0;
-  dim3 grid(pairs / MX_TM + n_experts, (width + 4 * MX_WAVE_COLS - 1) / (4 * MX_WAVE_COLS)), block(256);
+  const bool large = grouped_large(pairs, n_experts, pairs * ldh, 1ll * n_experts * width * ldw);
+  const int tile = large ? GT_ROWS : 64;
+  dim3 grid(pairs / tile + n_experts, (width + 4 * MX_WAVE_COLS - 1) / (4 * MX_WAVE_COLS)), block(256);
   PYLON_REQUIRE(grid.y <= 65535, "grouped_down: too many columns for one launch");
-  hipLaunchKernelGGL((grouped_rows_kernel<false, float>), grid, block, 0, stream, y, (long long)width,
-                     (const uint16_t*)hidden, ldh, nullptr, (const uint16_t*)w, ldw, (long long)width, offsets,
-                     n_experts, width, ff);
+  if (large)
+    hipLaunchKernelGGL((grouped_tiles_kernel<false, float>), grid, block, 0, stream, y, (long long)width,
+                       (const uint16_t*)hidden, ldh, nullptr, (const uint16_t*)w, ldw, (long long)width, offsets,
+                       n_experts, width, ff);
+  else
+    hipLaunchKernelGGL((grouped_rows_kernel<false, 4, float>), grid, block, 0, stream, y, (long long)width,
+                       (const uint16_t*)hidden, ldh, nullptr, (const uint16_t*)w, ldw, (long long)width, offsets,
+                       n_experts, width, ff);
   PYLON_LAUNCHED("grouped_down");
 }
 

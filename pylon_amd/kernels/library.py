@@ -59,7 +59,7 @@ _SIGNATURES = {
     "pylon_expert_gate_up": [P, P, I, L, P, I, L, P, I, I, I, I, P],
     "pylon_expert_down": [P, P, I, P, I, L, P, P, P, P, I, I, I, I, P],
     "pylon_softcap": [P, L, F, P],
-    "pylon_grouped_gate_up": [P, P, L, P, P, L, P, I, I, I, I, P],
+    "pylon_grouped_gate_up": [P, P, L, P, P, L, P, I, I, I, I, I, P],
     "pylon_grouped_down": [P, P, L, P, L, P, I, I, I, I, P],
     "pylon_expert_combine": [P, P, P, P, P, P, I, I, I, P],
 }

@@ -1220,7 +1220,8 @@ def experts_grouped(x: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, 
     place = torch.empty_like(order).scatter_(0, order, torch.arange(pairs, device=x.device)).to(torch.int32)
     hidden = torch.empty((pairs, ff), dtype=torch.bfloat16, device=x.device)
     _lib.call("pylon_grouped_gate_up", _dev(hidden, "hidden"), x.data_ptr(), x.stride(0), _dev(rows, "rows"),
-              gate_up.data_ptr(), gate_up.stride(0), _dev(offsets, "offsets"), pairs, n_experts, ff, width, _stream())
+              gate_up.data_ptr(), gate_up.stride(0), _dev(offsets, "offsets"), pairs, n_experts, ff, width, tokens,
+              _stream())
     y = torch.empty((pairs, width), dtype=torch.float32, device=x.device)
     _lib.call("pylon_grouped_down", _dev(y, "y"), _dev(hidden, "hidden"), ff, down.data_ptr(), down.stride(0),
               _dev(offsets, "offsets"), pairs, n_experts, ff, width, _stream())

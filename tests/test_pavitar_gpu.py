@@ -282,7 +282,7 @@ def test_mixture_of_experts_against_the_plain_one(ops, dtype, width, experts, to
         p["shared_gate_up"][shared:] = dev(w["f.shared.up"], dtype)
         p["shared_down"][:] = dev(w["f.shared.down"], dtype)
     mlp = {"router": {"experts": experts, "top": top}, "shared": None if shared is None else {"ff": shared}}
-    for n in (1, 5, 70, 150):  # the shared expert's products change kernels with the row count
+    for n in (1, 5, 70, 150, 400):  # the products change kernels with the row count (400: the experts' tiles through LDS)
         h = torch.tensor(rng.normal(size=(n, width)), dtype=dtype)
         want = plain.mixture(h.double().numpy(), w, "f.", mlp)
         got = part.forward(h.to(DEV), None)
