@@ -115,6 +115,74 @@ head_project_kernel(TX* __restrict__ out, const TX* __restrict__ x, long long x_
   }
 }
 
+// The same product for bfloat16 matrices whose rows are whole 16-byte pieces: a lane reads eight
+// neighbouring columns of a row of m[h] at once, sixteen lanes a 256-byte row segment, the sixteen
+// groups of lanes of a workgroup every sixteenth row; their sums meet by two shuffles inside a wave
+// and through LDS between the four waves, always in the same order.
+#define HW_COLS 128
+
+__global__ void __launch_bounds__(HP_THREADS)
+head_project_wide_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ x, long long x_stride,
+                         const bf16_t* __restrict__ m, const float* __restrict__ gate, int tokens, int heads, int n_in,
+                         int n_out) {
+  extern __shared__ float xs[];  // [HP_TOKENS, n_in], then the waves' partial sums [4, HP_TOKENS, HW_COLS]
+  float* partial = xs + HP_TOKENS * n_in;
+  const int t0 = blockIdx.x * HP_TOKENS, h = blockIdx.y, c0 = blockIdx.z * HW_COLS, tid = threadIdx.x;
+  for (int i = tid; i < HP_TOKENS * n_in; i += HP_THREADS) {
+    const int tt = i / n_in, k = i - tt * n_in;
+    xs[i] = (t0 + tt < tokens) ? to_float(x[static_cast<size_t>(t0 + tt) * x_stride + static_cast<size_t>(h) * n_in + k])
+                               : 0.f;
+  }
+  __syncthreads();
+  const int lane = tid & (PYLON_WAVE - 1), wave = tid / PYLON_WAVE;
+  const int cg = lane & 15, kg = wave * 4 + (lane >> 4);
+  float acc[HP_TOKENS][8];
+#pragma unroll
+  for (int tt = 0; tt < HP_TOKENS; ++tt)
+#pragma unroll
+    for (int c = 0; c < 8; ++c) acc[tt][c] = 0.f;
+  const int col = c0 + 8 * cg;
+  if (col < n_out) {  // n_out is a multiple of 8: the lane's eight columns are all inside
+    const bf16_t* mh = m + static_cast<size_t>(h) * n_in * n_out + col;
+#pragma unroll 4
+    for (int k = kg; k < n_in; k += 16) {
+      const uint4 raw = *reinterpret_cast<const uint4*>(mh + static_cast<size_t>(k) * n_out);
+      const uint32_t words[4] = {raw.x, raw.y, raw.z, raw.w};
+      float wv[8];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        wv[2 * j] = __uint_as_float(words[j] << 16);
+        wv[2 * j + 1] = __uint_as_float(words[j] & 0xffff0000u);
+      }
+#pragma unroll
+      for (int tt = 0; tt < HP_TOKENS; ++tt) {
+        const float xv = xs[tt * n_in + k];
+#pragma unroll
+        for (int c = 0; c < 8; ++c) acc[tt][c] = fmaf(xv, wv[c], acc[tt][c]);
+      }
+    }
+  }
+#pragma unroll
+  for (int tt = 0; tt < HP_TOKENS; ++tt)
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+      float v = acc[tt][c];
+      v += __shfl_xor(v, 16, PYLON_WAVE);
+      v += __shfl_xor(v, 32, PYLON_WAVE);
+      if (lane < 16) partial[(wave * HP_TOKENS + tt) * HW_COLS + 8 * cg + c] = v;
+    }
+  __syncthreads();
+  for (int i = tid; i < HP_TOKENS * HW_COLS; i += HP_THREADS) {
+    const int tt = i / HW_COLS, c = i % HW_COLS;
+    if (t0 + tt >= tokens || c0 + c >= n_out) continue;
+    float sum = partial[tt * HW_COLS + c];
+#pragma unroll
+    for (int wv = 1; wv < 4; ++wv) sum += partial[(wv * HP_TOKENS + tt) * HW_COLS + c];
+    const float g = gate != nullptr ? gate[static_cast<size_t>(t0 + tt) * heads + h] : 1.f;
+    out[(static_cast<size_t>(t0 + tt) * heads + h) * n_out + c0 + c] = from_float<bf16_t>(sum * g);
+  }
+}
+
 // x: [tokens, heads, n_in], rows x_stride elements apart; m: [heads, n_in, n_out]; gate: null or
 // float [tokens, heads]; out: [tokens, heads, n_out] of x's type.  m may be float while x is bfloat16.
 extern "C" int pylon_head_project(void* out, const void* x, int x_dtype, long long x_stride, const void* m,
@@ -128,6 +196,16 @@ extern "C" int pylon_head_project(void* out, const void* x, int x_dtype, long lo
   PYLON_REQUIRE(lds <= 64 * 1024, "head_project: %d inputs per head do not fit LDS", n_in);
   PYLON_REQUIRE(!(x_dtype == PYLON_F32 && m_dtype == PYLON_BF16), "head_project: float inputs take a float matrix");
   if (tokens == 0) return 0;
+  if (x_dtype == PYLON_BF16 && m_dtype == PYLON_BF16 && n_out % 8 == 0 && reinterpret_cast<uintptr_t>(m) % 16 == 0) {
+    const size_t wide_lds = sizeof(float) * (HP_TOKENS * n_in + 4 * HP_TOKENS * HW_COLS);
+    const int zw = (n_out + HW_COLS - 1) / HW_COLS;
+    if (wide_lds <= 64 * 1024 && zw <= 65535) {
+      hipLaunchKernelGGL(head_project_wide_kernel, dim3((tokens + HP_TOKENS - 1) / HP_TOKENS, heads, zw),
+                         dim3(HP_THREADS), wide_lds, stream, (bf16_t*)out, (const bf16_t*)x, x_stride,
+                         (const bf16_t*)m, gate, tokens, heads, n_in, n_out);
+      PYLON_LAUNCHED("head_project");
+    }
+  }
   const int zs = (n_out + HP_COLS - 1) / HP_COLS;
   PYLON_REQUIRE(zs <= 65535, "head_project: too many outputs per head for one launch");
   dim3 grid((tokens + HP_TOKENS - 1) / HP_TOKENS, heads, zs), block(HP_THREADS);
