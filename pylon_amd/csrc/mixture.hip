@@ -135,6 +135,48 @@ __device__ __forceinline__ float row_dot_share<bf16_t>(const bf16_t* __restrict_
   return acc;
 }
 
+// The lanes' shares of the dot products of ROWS bfloat16 rows with one vector in LDS, rows of a
+// multiple of 8 elements: every trip fetches two 16-byte pieces of every row before it multiplies
+// any, so that 2 ROWS loads of a wave are in flight together (one load at a time, a wave waits a
+// memory latency per kilobyte).  Every share is added up in the order of the row, as
+// row_dot_share adds it.
+template <int ROWS>
+__device__ __forceinline__ void rows_dot_share(const bf16_t* const (&rows)[ROWS], const float* __restrict__ xs, int n,
+                                               int lane, float (&acc)[ROWS]) {
+  constexpr int STEP = PYLON_WAVE * 8;
+  for (int i = lane * 8; i < n; i += 2 * STEP) {
+    const bool second = i + STEP < n;
+    uint4 raw[ROWS][2];
+#pragma unroll
+    for (int q = 0; q < ROWS; ++q) {
+      raw[q][0] = *reinterpret_cast<const uint4*>(rows[q] + i);
+      raw[q][1] = second ? *reinterpret_cast<const uint4*>(rows[q] + i + STEP) : uint4{0u, 0u, 0u, 0u};
+    }
+#pragma unroll
+    for (int q = 0; q < ROWS; ++q)
+#pragma unroll
+      for (int p = 0; p < 2; ++p) {
+        if (p == 1 && !second) continue;
+        const float* xv = xs + i + p * STEP;
+        const uint32_t w[4] = {raw[q][p].x, raw[q][p].y, raw[q][p].z, raw[q][p].w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          acc[q] = fmaf(xv[2 * j], __uint_as_float(w[j] << 16), acc[q]);
+          acc[q] = fmaf(xv[2 * j + 1], __uint_as_float(w[j] & 0xffff0000u), acc[q]);
+        }
+      }
+  }
+}
+
+template <typename T>
+struct is_bf16 {
+  static constexpr bool value = false;
+};
+template <>
+struct is_bf16<bf16_t> {
+  static constexpr bool value = true;
+};
+
 template <typename TX, typename TW>
 __global__ void __launch_bounds__(256)
 expert_gate_up_kernel(TX* __restrict__ hidden, const TX* __restrict__ x, long long x_stride,
@@ -150,10 +192,34 @@ expert_gate_up_kernel(TX* __restrict__ hidden, const TX* __restrict__ x, long lo
   const TW* up = gate + static_cast<size_t>(ff) * w_stride;
   const int j0 = blockIdx.x * units_per_block;
   const int j1 = j0 + units_per_block < ff ? j0 + units_per_block : ff;
-  for (int j = j0 + wave; j < j1; j += 4) {
-    const float g = wave_sum(row_dot_share<TW>(gate + static_cast<size_t>(j) * w_stride, xs, width, lane, wide));
-    const float u = wave_sum(row_dot_share<TW>(up + static_cast<size_t>(j) * w_stride, xs, width, lane, wide));
-    if (lane == 0) hidden[static_cast<size_t>(pair) * ff + j] = from_float<TX>(g / (1.0f + expf(-g)) * u);
+  // a wave takes two hidden units at a time: the lanes' shares of all four rows first (their loads
+  // are in flight together), then the four sums over the lanes
+  for (int j = j0 + 2 * wave; j < j1; j += 8) {
+    const bool two = j + 1 < j1;
+    float gs0, us0, gs1, us1;
+    bool done = false;
+    if constexpr (is_bf16<TW>::value) {
+      if (wide) {  // all four rows together (a lone last unit twice: its second result is dropped)
+        const int k = two ? j + 1 : j;
+        const bf16_t* const rows[4] = {gate + static_cast<size_t>(j) * w_stride, up + static_cast<size_t>(j) * w_stride,
+                                       gate + static_cast<size_t>(k) * w_stride, up + static_cast<size_t>(k) * w_stride};
+        float acc[4] = {0.f, 0.f, 0.f, 0.f};
+        rows_dot_share<4>(rows, xs, width, lane, acc);
+        gs0 = acc[0], us0 = acc[1], gs1 = acc[2], us1 = acc[3];
+        done = true;
+      }
+    }
+    if (!done) {
+      gs0 = row_dot_share<TW>(gate + static_cast<size_t>(j) * w_stride, xs, width, lane, wide);
+      us0 = row_dot_share<TW>(up + static_cast<size_t>(j) * w_stride, xs, width, lane, wide);
+      gs1 = two ? row_dot_share<TW>(gate + static_cast<size_t>(j + 1) * w_stride, xs, width, lane, wide) : 0.f;
+      us1 = two ? row_dot_share<TW>(up + static_cast<size_t>(j + 1) * w_stride, xs, width, lane, wide) : 0.f;
+    }
+    const float g0 = wave_sum(gs0), u0 = wave_sum(us0), g1 = wave_sum(gs1), u1 = wave_sum(us1);
+    if (lane == 0) {
+      hidden[static_cast<size_t>(pair) * ff + j] = from_float<TX>(g0 / (1.0f + expf(-g0)) * u0);
+      if (two) hidden[static_cast<size_t>(pair) * ff + j + 1] = from_float<TX>(g1 / (1.0f + expf(-g1)) * u1);
+    }
   }
 }
 
@@ -172,7 +238,7 @@ extern "C" int pylon_expert_gate_up(void* hidden, const void* x, int x_dtype, lo
   if (tokens == 0) return 0;
   const int per = w_dtype == PYLON_F32 ? 4 : 8;
   const int wide = (width % per == 0 && w_stride % per == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0) ? 1 : 0;
-  const int units = 16;
+  const int units = 32;
   // grid.y is limited to 65535: more pairs go in several launches of whole tokens
   const long long pairs = static_cast<long long>(tokens) * top;
   const long long per_launch = static_cast<long long>(65535 / top) * top;
@@ -205,14 +271,50 @@ expert_down_kernel(float* __restrict__ out, const TH* __restrict__ hidden, const
   __syncthreads();
   const int c0 = blockIdx.x * cols_per_block;
   const int c1 = c0 + cols_per_block < width ? c0 + cols_per_block : width;
+  if constexpr (is_bf16<TW>::value) {
+    if (wide && cols_per_block == 16) {
+      // a wave takes four neighbouring columns: per chosen expert the lanes' shares of its four rows
+      // with all their loads in flight together, weighed in the order of the token's choices; one sum
+      // over the lanes per column at the end
+      const int c = c0 + 4 * wave;
+      if (c >= c1) return;
+      float share[4] = {0.f, 0.f, 0.f, 0.f};
+      for (int s = 0; s < top; ++s) {
+        const int e = experts[static_cast<size_t>(t) * top + s];
+        const bf16_t* base = w + static_cast<size_t>(e) * width * w_stride;
+        const bf16_t* rows[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) rows[q] = base + static_cast<size_t>(c + q < c1 ? c + q : c1 - 1) * w_stride;
+        float part[4] = {0.f, 0.f, 0.f, 0.f};
+        rows_dot_share<4>(rows, hs + s * ff, ff, lane, part);
+        const float weight = weights[static_cast<size_t>(t) * top + s];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) share[q] = fmaf(weight, part[q], share[q]);
+      }
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        float acc = wave_sum(share[q]);
+        if (lane == 0 && c + q < c1) {
+          if (shared != nullptr) {
+            const float g = shared_gate != nullptr ? shared_gate[t] : 1.f;
+            acc = fmaf(g, shared[static_cast<size_t>(t) * width + c + q], acc);
+          }
+          out[static_cast<size_t>(t) * width + c + q] = acc;
+        }
+      }
+      return;
+    }
+  }
   for (int c = c0 + wave; c < c1; c += 4) {
-    float acc = 0.f;
+    // every lane weighs its shares of the chosen experts' rows, in the order of the token's choices;
+    // one sum over the lanes at the end
+    float share = 0.f;
     for (int s = 0; s < top; ++s) {
       const int e = experts[static_cast<size_t>(t) * top + s];
       const TW* row = w + (static_cast<size_t>(e) * width + c) * w_stride;
-      acc = fmaf(weights[static_cast<size_t>(t) * top + s], wave_sum(row_dot_share<TW>(row, hs + s * ff, ff, lane, wide)),
-                 acc);
+      share = fmaf(weights[static_cast<size_t>(t) * top + s], row_dot_share<TW>(row, hs + s * ff, ff, lane, wide), share);
     }
+    float acc = wave_sum(share);
     if (lane == 0) {
       if (shared != nullptr) {
         const float g = shared_gate != nullptr ? shared_gate[t] : 1.f;
