@@ -474,7 +474,7 @@ grouped_rows_kernel(TO* __restrict__ out, long long ldo, const uint16_t* __restr
 #define GT_PITCH 144
 
 template <bool GLU, typename TO>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(256, 2)
 grouped_tiles_kernel(TO* __restrict__ out, long long ldo, const uint16_t* __restrict__ x, long long ldx,
                      const int* __restrict__ row_index, const uint16_t* __restrict__ w, long long ldw,
                      long long expert_rows, const int* __restrict__ offsets, int n_experts, int N, int K) {
