@@ -462,12 +462,13 @@ grouped_rows_kernel(TO* __restrict__ out, long long ldo, const uint16_t* __restr
   }
 }
 
-// The same product for experts with many pairs each: tiles of 128 pairs x 128 output columns
+// The same product for experts with many pairs each: tiles of 128 pairs x 256 output columns
 // (with the gated epilogue: 128 gate and their 128 up columns), K in pieces of 64 elements that all
 // 256 threads bring into LDS together, whole 128-byte row segments at a time (a thread 16 bytes of
 // one row; 32 rows further on its next load), the next piece on its way into registers while the
 // matrix instructions read the current one from LDS.  Rows lie 144 bytes apart in LDS, so that
-// the 16 rows of an operand fall into different banks.  A wave takes all 128 rows and 32 columns.
+// the 16 rows of an operand fall into different banks.  A wave takes all 128 rows and a quarter of
+// the columns; the 16-row pieces past a tile's last pair are not multiplied.
 #define GT_ROWS 128
 #define GT_COLS 128
 #define GT_K 64
@@ -478,9 +479,10 @@ __global__ void __launch_bounds__(256, 2)
 grouped_tiles_kernel(TO* __restrict__ out, long long ldo, const uint16_t* __restrict__ x, long long ldx,
                      const int* __restrict__ row_index, const uint16_t* __restrict__ w, long long ldw,
                      long long expert_rows, const int* __restrict__ offsets, int n_experts, int N, int K) {
-  constexpr int WROWS = GLU ? 2 * GT_COLS : GT_COLS;
+  constexpr int WROWS = 2 * GT_COLS;  // GLU: 128 gate rows and their 128 up rows; else 256 output columns
+  constexpr int TILE_COLS = GLU ? GT_COLS : 2 * GT_COLS, WAVE_COLS = TILE_COLS / 4;
   constexpr int XLOADS = GT_ROWS / 32, LOADS = (GT_ROWS + WROWS) / 32;
-  constexpr int J = GLU ? 4 : 2, MT = GT_ROWS / 16;
+  constexpr int J = 4, MT = GT_ROWS / 16;
   __shared__ __attribute__((aligned(16))) unsigned char lds[(GT_ROWS + WROWS) * GT_PITCH];
   const int tid = threadIdx.x, lane = tid & (PYLON_WAVE - 1), wave = tid / PYLON_WAVE;
   const int r = lane & 15, g = lane >> 4;
@@ -496,7 +498,7 @@ grouped_tiles_kernel(TO* __restrict__ out, long long ldo, const uint16_t* __rest
     tile -= tiles;
   }
   if (e == n_experts) return;  // the whole workgroup: no barrier is missed
-  const int n0 = blockIdx.y * GT_COLS;
+  const int n0 = blockIdx.y * TILE_COLS;
 
   // what this thread brings: the 16-byte piece `piece` of rows lrow, lrow + 32, ... of the tile in LDS
   const int piece = tid & 7, lrow = tid >> 3;
@@ -539,11 +541,13 @@ grouped_tiles_kernel(TO* __restrict__ out, long long ldo, const uint16_t* __rest
       mx_bf16x8 wf[J];
 #pragma unroll
       for (int j = 0; j < J; ++j) {
-        const int row = GT_ROWS + (GLU && j >= 2 ? GT_COLS : 0) + wave * 32 + 16 * (j & 1) + r;
+        const int row = GLU ? GT_ROWS + (j >= 2 ? GT_COLS : 0) + wave * 32 + 16 * (j & 1) + r
+                            : GT_ROWS + wave * WAVE_COLS + 16 * j + r;
         wf[j] = *reinterpret_cast<const mx_bf16x8*>(lds + row * GT_PITCH + h * 64 + g * 16);
       }
 #pragma unroll
       for (int t = 0; t < MT; ++t) {
+        if (16 * t >= rows) continue;  // a tile's last rows: nothing to multiply (the same for the whole workgroup)
         const mx_bf16x8 xf = *reinterpret_cast<const mx_bf16x8*>(lds + (16 * t + r) * GT_PITCH + h * 64 + g * 16);
 #pragma unroll
         for (int j = 0; j < J; ++j) acc[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[j], xf, acc[j][t], 0, 0, 0);
@@ -551,16 +555,17 @@ grouped_tiles_kernel(TO* __restrict__ out, long long ldo, const uint16_t* __rest
     }
     __syncthreads();
   }
-  // acc[j][t][i] is the sum for row 16 t + r and column n0 + 32 wave + 16 (j & 1) + 4 g + i
+  // acc[j][t][i] is the sum for row 16 t + r and, gated, column n0 + 32 wave + 16 (j & 1) + 4 g + i
+  // (j < 2 the gate's, j >= 2 the up's), else column n0 + 64 wave + 16 j + 4 g + i
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
     if (16 * t + r >= rows) continue;
     TO* orow = out + static_cast<size_t>(row0 + 16 * t + r) * ldo;
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < (GLU ? 2 : J); ++j)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int n = n0 + 32 * wave + 16 * j + 4 * g + i;
+        const int n = n0 + WAVE_COLS * wave + 16 * j + 4 * g + i;
         if (n >= N) continue;
         float v = acc[j][t][i];
         if constexpr (GLU) v = v / (1.0f + expf(-v)) * acc[2 + j][t][i];
@@ -617,8 +622,8 @@ extern "C" int pylon_grouped_down(float* y, const void* hidden, long long ldh, c
   if (grouped_checks("grouped_down", hidden, ldh, w, ldw, ff, width, pairs, n_experts)) return 1;
   if (pairs == 0) return 0;
   const bool large = grouped_large(pairs, n_experts, pairs * ldh, 1ll * n_experts * width * ldw);
-  const int tile = large ? GT_ROWS : 64;
-  dim3 grid(pairs / tile + n_experts, (width + 4 * MX_WAVE_COLS - 1) / (4 * MX_WAVE_COLS)), block(256);
+  const int tile = large ? GT_ROWS : 64, cols = large ? 2 * GT_COLS : 4 * MX_WAVE_COLS;
+  dim3 grid(pairs / tile + n_experts, (width + cols - 1) / cols), block(256);
   PYLON_REQUIRE(grid.y <= 65535, "grouped_down: too many columns for one launch");
   if (large)
     hipLaunchKernelGGL((grouped_tiles_kernel<false, float>), grid, block, 0, stream, y, (long long)width,

@@ -119,6 +119,9 @@ class StepContext:
     logits_out: Optional[torch.Tensor] = None  # float32 [>= n_logits, vocab]: where the logits go, if given
     arena: Optional[MetadataArena] = None  # pinned staging for what parts put on the device themselves
     _tiles: Dict[Tuple[int, int, int], torch.Tensor] = field(default_factory=dict)
+    # what a part has derived from the step's metadata and layers of its kind can share (by a key of
+    # the part's choosing): made once a step instead of once a layer
+    memo: Dict[object, object] = field(default_factory=dict)
 
     def cache(self, cache_id: int) -> CacheView:
         return self.views[cache_id]

@@ -116,8 +116,10 @@ class LatentAttention(Part):
             repeat = heads // group
             positions, rows = ctx.positions, None
             if repeat > 1:  # every group of heads a query token of its own, on its request's row of the table
-                positions = ctx.positions.repeat_interleave(repeat)
-                rows = ctx.tok_row.repeat_interleave(repeat)
+                key = ("latent_attention.groups", repeat)
+                if key not in ctx.memo:  # once a step, not once a layer
+                    ctx.memo[key] = (ctx.positions.repeat_interleave(repeat), ctx.tok_row.repeat_interleave(repeat))
+                positions, rows = ctx.memo[key]
             cuts, splits = self._decode_launch(tokens * repeat, self._span(ctx.max_len))
             mixed = ops.attention_decode(
                 q.view(tokens * repeat, group, rank), latents, latents, cache.block_table, rows, positions,
