@@ -294,6 +294,37 @@ def test_mixture_of_experts_against_the_plain_one(ops, dtype, width, experts, to
                 assert np.abs(alone.cpu().numpy() - got[3:4].cpu().numpy()).max() <= 2e-5 * np.abs(want).max()
 
 
+@pytest.mark.parametrize("tokens", [300, 400])
+def test_experts_sorted_by_expert_agree_with_token_by_token_at_tile_edges(ops, tokens):
+    """The matrix-core path (pairs sorted by expert; tiles of 64 rows at 300 tokens, of 128 through LDS
+    at 400) against the token-by-token kernels on routings made by hand: an expert nobody chose, experts
+    with exactly one tile, one pair more, one pair, and the rest."""
+    rng = np.random.default_rng(tokens)
+    width, ff, experts, top = 72, 40, 5, 2
+    pairs = tokens * top
+    tile = 128 if pairs // experts >= 128 else 64
+    counts = [0, tile, tile + 1, 1]
+    counts.append(pairs - sum(counts))
+    flat = np.repeat(np.arange(experts), counts)
+    rng.shuffle(flat)  # (a token may meet an expert twice here, which a router never does and the kernels do not mind)
+    chosen = flat.reshape(tokens, top)
+    weights = rng.uniform(0.1, 1.0, size=(tokens, top)).astype(np.float32)
+    x = torch.tensor(rng.normal(size=(tokens, width)), dtype=torch.bfloat16, device=DEV)
+    gate_up = torch.tensor(rng.normal(size=(experts * 2 * ff, width)) * 0.2, dtype=torch.bfloat16, device=DEV)
+    down = torch.tensor(rng.normal(size=(experts * width, ff)) * 0.2, dtype=torch.bfloat16, device=DEV)
+    shared = torch.tensor(rng.normal(size=(tokens, width)), dtype=torch.float32, device=DEV)
+    gate = torch.tensor(rng.uniform(size=tokens), dtype=torch.float32, device=DEV)
+    e, w = i32(chosen.reshape(-1)).view(tokens, top), dev(weights)
+    hidden = ops.expert_gate_up(x, gate_up, e, n_experts=experts, ff=ff)
+    want = ops.expert_down(hidden, down, e, w, n_experts=experts, width=width, shared=shared, shared_gate=gate)
+    got = ops.experts_grouped(x, gate_up, down, e, w, n_experts=experts, ff=ff, shared=shared, shared_gate=gate)
+    close(got.cpu().numpy(), want.double().cpu().numpy(), 2e-2, "sorted by expert")
+    # and without a shared expert
+    want = ops.expert_down(hidden, down, e, w, n_experts=experts, width=width)
+    got = ops.experts_grouped(x, gate_up, down, e, w, n_experts=experts, ff=ff)
+    close(got.cpu().numpy(), want.double().cpu().numpy(), 2e-2, "sorted by expert, no shared expert")
+
+
 def test_soft_cap(ops):
     x = torch.tensor([[-1e4, -30.0, -1.0, 0.0, 0.5, 29.0, 1e4]], device=DEV)
     want = 15.0 * np.tanh(x.double().cpu().numpy() / 15.0)
