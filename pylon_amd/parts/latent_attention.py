@@ -111,9 +111,10 @@ class LatentAttention(Part):
         q = ops.head_project(q.view(tokens, heads, spec.head_dim), self.params["uk"].view(heads, spec.head_dim, rank))
         mask = dict(window=spec.window, chunk=spec.chunk)
         latents = cache.k  # [pages, page_size, 1, kv_rank]: keys and values at once
-        if self._matrix_cores() and q.dtype == latents.dtype and ctx.decode_only and tokens <= ops.DECODE_MAX_TOKENS:
-            group = self._group()
-            repeat = heads // group
+        group = self._group()
+        repeat = heads // group
+        if self._matrix_cores() and q.dtype == latents.dtype and ctx.decode_only \
+                and tokens * repeat <= ops.DECODE_MAX_TOKENS:
             positions, rows = ctx.positions, None
             if repeat > 1:  # every group of heads a query token of its own, on its request's row of the table
                 key = ("latent_attention.groups", repeat)
